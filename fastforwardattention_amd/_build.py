@@ -1,0 +1,81 @@
+"""Build recipe for the native parts (run here on CPU; hipcc cross-compiles gfx950).
+
+  libffa_hip.so        C ABI + gfx950 kernels            hipcc  (csrc/*.hip, csrc/*.cpp)
+  ff_attention*.so     pybind11 torch extension          g++    (csrc/torch_ffa_api.cpp)
+
+Counterpart of the reference's setup.py:4-16 (CUDAExtension) and compile.sh:6-9
+(libffa.so).  Both artefacts are written next to this file so that they travel with the
+source tree; nothing is installed into site-packages.
+
+    python -m fastforwardattention_amd._build            # build everything
+    python -m fastforwardattention_amd._build --lib      # C-ABI library only
+"""
+from __future__ import annotations
+
+import os
+import subprocess
+import sys
+import sysconfig
+from pathlib import Path
+
+PKG_DIR = Path(__file__).resolve().parent
+CSRC = PKG_DIR / "csrc"
+INCLUDE = PKG_DIR.parent / "include"
+LIB_PATH = PKG_DIR / "libffa_hip.so"
+EXT_SUFFIX = sysconfig.get_config_var("EXT_SUFFIX") or ".so"
+EXT_PATH = PKG_DIR / f"ff_attention{EXT_SUFFIX}"
+ROCM = Path(os.environ.get("ROCM_PATH", "/opt/rocm"))
+
+HIP_ARCH = "gfx950"
+# -packed-fp32-ops off: keep the compiler from forming v_pk_*_f32.
+HIPCC_FLAGS = [
+    f"--offload-arch={HIP_ARCH}", "-O3", "-std=c++17", "-fPIC", "-shared",
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-Wall", "-Wno-unused-function",
+]
+
+
+def _run(cmd):
+    print("+", " ".join(str(c) for c in cmd), flush=True)
+    subprocess.run([str(c) for c in cmd], check=True)
+
+
+def build_lib() -> Path:
+    srcs = [CSRC / "ffa_kernels.hip", CSRC / "ffa_api.cpp", CSRC / "ffa_plan.cpp"]
+    hipcc = ROCM / "bin" / "hipcc"
+    _run([hipcc, *HIPCC_FLAGS, f"-I{INCLUDE}", f"-I{CSRC}", *srcs, "-o", LIB_PATH])
+    return LIB_PATH
+
+
+def build_ext() -> Path:
+    import torch
+    from torch.utils import cpp_extension as ce
+
+    inc = [f"-I{p}" for p in ce.include_paths()] + [
+        f"-I{sysconfig.get_paths()['include']}", f"-I{INCLUDE}", f"-I{ROCM / 'include'}"]
+    torch_lib = Path(torch.__file__).resolve().parent / "lib"
+    abi = int(torch._C._GLIBCXX_USE_CXX11_ABI)
+    cmd = ["g++", "-O2", "-std=c++17", "-fPIC", "-shared", "-fvisibility=hidden",
+           "-D__HIP_PLATFORM_AMD__=1", "-DUSE_ROCM=1", f"-D_GLIBCXX_USE_CXX11_ABI={abi}",
+           "-DTORCH_EXTENSION_NAME=ff_attention", "-DTORCH_API_INCLUDE_EXTENSION_H",
+           *inc, CSRC / "torch_ffa_api.cpp", "-o", EXT_PATH,
+           f"-L{torch_lib}", f"-L{PKG_DIR}", f"-L{ROCM / 'lib'}",
+           "-lc10", "-lc10_hip", "-ltorch", "-ltorch_cpu", "-ltorch_hip", "-ltorch_python",
+           "-lffa_hip", "-lamdhip64",
+           "-Wl,-rpath,$ORIGIN", f"-Wl,-rpath,{torch_lib}", f"-Wl,-rpath,{ROCM / 'lib'}"]
+    _run(cmd)
+    return EXT_PATH
+
+
+def build_all() -> None:
+    build_lib()
+    build_ext()
+
+
+if __name__ == "__main__":
+    if "--lib" in sys.argv:
+        build_lib()
+    elif "--ext" in sys.argv:
+        build_ext()
+    else:
+        build_all()

@@ -1,0 +1,183 @@
+// C ABI of the decode-attention engine: argument validation, planning, workspace carving.
+// Pure host C++ (no device code, no HIP headers); the launchers live in ffa_kernels.hip.
+#include <math.h>
+#include <stdint.h>
+
+#include "ffa_c_api.h"
+#include "ffa_host.h"
+
+using namespace ffa;
+
+namespace {
+
+bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+int validate_decode(const DecodeArgs& a) {
+    if (a.precision != FFA_PRECISION_F16 && a.precision != FFA_PRECISION_F32) return FFA_ERR_DTYPE;
+    if (a.Dh != 64 && a.Dh != 128 && a.Dh != 256) return FFA_ERR_HEAD_DIM;
+    if (a.B <= 0 || a.H <= 0 || a.Lmax <= 0) return FFA_ERR_SHAPE;
+    if ((long long)a.B * a.H > (1ll << 24)) return FFA_ERR_SHAPE;
+    if (a.t < 0 || a.t >= a.Lmax) return FFA_ERR_TIMESTEP;
+    if (!(a.p >= 0.f) || isinf(a.p)) return FFA_ERR_PROB_THRESH;
+    if (!a.q || !a.k || !a.v || !a.k_cache || !a.v_cache || !a.out) return FFA_ERR_NULL_POINTER;
+    if (!aligned16(a.q) || !aligned16(a.k) || !aligned16(a.v) || !aligned16(a.k_cache) ||
+        !aligned16(a.v_cache) || !aligned16(a.out))
+        return FFA_ERR_ALIGNMENT;
+    return FFA_OK;
+}
+
+int run_decode(const DecodeArgs& a, const ffa_launch_plan* user_plan, void* workspace,
+               size_t workspace_bytes) {
+    int st = validate_decode(a);
+    if (st != FFA_OK) return st;
+    const bool diag = a.kept_count != nullptr || a.skip_mask != nullptr;
+
+    ffa_launch_plan plan;
+    if (user_plan != nullptr) {
+        plan = *user_plan;
+    } else {
+        // Diagnostics exist only in the one-workgroup kernel.
+        st = plan_launch(a.precision, a.B, a.H, a.Dh, a.t, a.p, /*use_default=*/0,
+                         diag ? 256 : query_compute_units(), &plan);
+        if (st == FFA_OK && diag && plan.kind != FFA_LAUNCH_WORKGROUP)
+            st = plan_launch(a.precision, a.B, a.H, a.Dh, a.t, 1.f, 0, 256, &plan);
+        if (st != FFA_OK) return st;
+    }
+    st = validate_plan(plan, a.precision, a.t, a.p);
+    if (st != FFA_OK) return st;
+    if (diag && plan.kind != FFA_LAUNCH_WORKGROUP) return FFA_ERR_PLAN;
+
+    WorkspaceView ws = {nullptr, nullptr, nullptr};
+    if (plan.kind == FFA_LAUNCH_SPLIT && plan.n_splits > 1) {
+        const int bh = a.B * a.H;
+        if (workspace == nullptr || workspace_bytes < workspace_bytes_for(bh, a.Dh, plan.n_splits))
+            return FFA_ERR_WORKSPACE;
+        if (!aligned16(workspace)) return FFA_ERR_ALIGNMENT;
+        char* base = static_cast<char*>(workspace);
+        ws.cnt = reinterpret_cast<unsigned int*>(base);
+        ws.ml = reinterpret_cast<float*>(base + workspace_counter_bytes(bh));
+        ws.acc = reinterpret_cast<float*>(base + workspace_counter_bytes(bh) +
+                                          align_up((size_t)bh * plan.n_splits * 2 * sizeof(float), 256));
+    }
+    return launch_decode(a, plan, ws);
+}
+
+int run_init_cache(int precision, void* k_dst, void* v_dst, const void* k_src, const void* v_src,
+                   int B, int L, int Lmax, int Dh, int H, void* stream) {
+    if (Dh != 64 && Dh != 128 && Dh != 256) return FFA_ERR_HEAD_DIM;
+    if (B <= 0 || H <= 0 || L < 0 || Lmax <= 0 || L > Lmax) return FFA_ERR_SHAPE;
+    if (!k_dst || !v_dst) return FFA_ERR_NULL_POINTER;
+    if (L == 0) return FFA_OK;
+    if (!k_src || !v_src) return FFA_ERR_NULL_POINTER;
+    if (!aligned16(k_dst) || !aligned16(v_dst) || !aligned16(k_src) || !aligned16(v_src))
+        return FFA_ERR_ALIGNMENT;
+    return launch_init_cache(precision, k_dst, v_dst, k_src, v_src, B, H, L, Lmax, Dh, stream);
+}
+
+}  // namespace
+
+extern "C" {
+
+int ffa_api_version(void) { return FFA_API_VERSION; }
+
+const char* ffa_status_string(int status) {
+    switch (status) {
+        case FFA_OK: return "ok";
+        case FFA_ERR_NULL_POINTER: return "a required pointer is NULL";
+        case FFA_ERR_DTYPE: return "unsupported precision (expected 16 or 32)";
+        case FFA_ERR_HEAD_DIM: return "unsupported head dimension (expected 64, 128 or 256)";
+        case FFA_ERR_SHAPE: return "invalid batch, head or sequence size";
+        case FFA_ERR_TIMESTEP: return "timestep outside [0, max_seq_len)";
+        case FFA_ERR_ALIGNMENT: return "pointer is not 16-byte aligned";
+        case FFA_ERR_WORKSPACE: return "workspace missing or too small for the launch plan";
+        case FFA_ERR_PLAN: return "malformed launch plan";
+        case FFA_ERR_TOO_LONG: return "sequence too long for a one-workgroup launch";
+        case FFA_ERR_PROB_THRESH: return "prob_thresh must be a finite number >= 0";
+        case FFA_ERR_LAUNCH: return "HIP kernel launch failed";
+        case FFA_ERR_NO_DEVICE: return "no usable HIP device";
+        default: return "unknown status";
+    }
+}
+
+int ffa_device_compute_units(void) { return query_compute_units(); }
+
+int ffa_plan_launch(int precision, int batch_size, int head_num, int head_dim, int t,
+                    float prob_thresh, int use_default_kernel_launch, int compute_units,
+                    ffa_launch_plan* plan) {
+    if (compute_units <= 0 && !use_default_kernel_launch) {
+        compute_units = query_compute_units();
+        if (compute_units <= 0) return FFA_ERR_NO_DEVICE;
+    }
+    return plan_launch(precision, batch_size, head_num, head_dim, t, prob_thresh,
+                       use_default_kernel_launch, compute_units, plan);
+}
+
+size_t ffa_workspace_bytes(int batch_size, int head_num, int head_dim, int max_seq_len) {
+    if (batch_size <= 0 || head_num <= 0 || head_dim <= 0 || max_seq_len <= 0) return 0;
+    const int bh = batch_size * head_num;
+    return workspace_bytes_for(bh, head_dim, max_splits_for(bh, max_seq_len));
+}
+
+int ffa_workspace_init(void* workspace, size_t workspace_bytes, void* stream) {
+    if (workspace == nullptr) return FFA_ERR_NULL_POINTER;
+    if (!aligned16(workspace)) return FFA_ERR_ALIGNMENT;
+    return launch_fill_u32(static_cast<unsigned int*>(workspace), workspace_bytes / 4, 0u, stream);
+}
+
+int ffa_init_cache_f16(uint16_t* k_dst, uint16_t* v_dst, const uint16_t* k_src,
+                       const uint16_t* v_src, int batch_size, int seq_len, int max_seq_len,
+                       int head_dim, int head_num, void* stream) {
+    return run_init_cache(FFA_PRECISION_F16, k_dst, v_dst, k_src, v_src, batch_size, seq_len,
+                          max_seq_len, head_dim, head_num, stream);
+}
+
+int ffa_init_cache_f32(float* k_dst, float* v_dst, const float* k_src, const float* v_src,
+                       int batch_size, int seq_len, int max_seq_len, int head_dim, int head_num,
+                       void* stream) {
+    return run_init_cache(FFA_PRECISION_F32, k_dst, v_dst, k_src, v_src, batch_size, seq_len,
+                          max_seq_len, head_dim, head_num, stream);
+}
+
+int ffa_attention_diag(int precision, int batch_size, int head_num, int head_dim, int max_seq_len,
+                       float softmax_scale, int t, const void* q, const void* k, const void* v,
+                       void* k_cache, void* v_cache, void* out, const int* seq_lengths,
+                       float prob_thresh, const ffa_launch_plan* plan, int right_or_no_padding,
+                       void* workspace, size_t workspace_bytes, uint32_t* kept_count,
+                       uint8_t* skip_mask, void* stream) {
+    DecodeArgs a;
+    a.precision = precision;
+    a.B = batch_size; a.H = head_num; a.Dh = head_dim; a.Lmax = max_seq_len; a.t = t;
+    a.scale = softmax_scale; a.p = prob_thresh;
+    a.q = q; a.k = k; a.v = v;
+    a.k_cache = k_cache; a.v_cache = v_cache; a.out = out;
+    a.seq_lengths = seq_lengths;
+    a.right_or_no_padding = right_or_no_padding;
+    a.kept_count = kept_count; a.skip_mask = skip_mask;
+    a.stream = stream;
+    return run_decode(a, plan, workspace, workspace_bytes);
+}
+
+int ffa_attention_f16(int batch_size, int head_num, int head_dim, int max_seq_len,
+                      float softmax_scale, int t, const uint16_t* q, const uint16_t* k,
+                      const uint16_t* v, uint16_t* k_cache, uint16_t* v_cache, uint16_t* out,
+                      const int* seq_lengths, float prob_thresh, const ffa_launch_plan* plan,
+                      int right_or_no_padding, void* workspace, size_t workspace_bytes,
+                      void* stream) {
+    return ffa_attention_diag(FFA_PRECISION_F16, batch_size, head_num, head_dim, max_seq_len,
+                              softmax_scale, t, q, k, v, k_cache, v_cache, out, seq_lengths,
+                              prob_thresh, plan, right_or_no_padding, workspace, workspace_bytes,
+                              nullptr, nullptr, stream);
+}
+
+int ffa_attention_f32(int batch_size, int head_num, int head_dim, int max_seq_len,
+                      float softmax_scale, int t, const float* q, const float* k, const float* v,
+                      float* k_cache, float* v_cache, float* out, const int* seq_lengths,
+                      float prob_thresh, const ffa_launch_plan* plan, int right_or_no_padding,
+                      void* workspace, size_t workspace_bytes, void* stream) {
+    return ffa_attention_diag(FFA_PRECISION_F32, batch_size, head_num, head_dim, max_seq_len,
+                              softmax_scale, t, q, k, v, k_cache, v_cache, out, seq_lengths,
+                              prob_thresh, plan, right_or_no_padding, workspace, workspace_bytes,
+                              nullptr, nullptr, stream);
+}
+
+}  // extern "C"

@@ -1,0 +1,117 @@
+// Device-side building blocks for the gfx950 decode-attention kernels:
+// wave64 DPP reductions, 16-byte chunk dot/fma for fp16 and fp32, fp16 rounding helpers.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace ffa {
+
+typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+
+constexpr int kWave = 64;
+constexpr float kLog2e = 1.4426950408889634f;
+
+// ---------------------------------------------------------------------------------------
+// DPP lane exchange.  ctrl values: quad_perm [1,0,3,2] = 0xB1, [2,3,0,1] = 0x4E,
+// row_half_mirror = 0x141, row_mirror = 0x140.  After the four steps every lane of a
+// 16-lane row holds that row's reduction; the four rows are merged through readlane.
+template <int CTRL>
+__device__ __forceinline__ float dpp_f32(float x) {
+    return __builtin_bit_cast(
+        float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), CTRL, 0xf, 0xf, false));
+}
+
+__device__ __forceinline__ float wave_max(float x) {
+    x = fmaxf(x, dpp_f32<0xB1>(x));
+    x = fmaxf(x, dpp_f32<0x4E>(x));
+    x = fmaxf(x, dpp_f32<0x141>(x));
+    x = fmaxf(x, dpp_f32<0x140>(x));
+    const float a = __builtin_amdgcn_readlane(x, 0), b = __builtin_amdgcn_readlane(x, 16);
+    const float c = __builtin_amdgcn_readlane(x, 32), d = __builtin_amdgcn_readlane(x, 48);
+    return fmaxf(fmaxf(a, b), fmaxf(c, d));
+}
+
+__device__ __forceinline__ float wave_sum(float x) {
+    x += dpp_f32<0xB1>(x);
+    x += dpp_f32<0x4E>(x);
+    x += dpp_f32<0x141>(x);
+    x += dpp_f32<0x140>(x);
+    const float a = __builtin_amdgcn_readlane(x, 0), b = __builtin_amdgcn_readlane(x, 16);
+    const float c = __builtin_amdgcn_readlane(x, 32), d = __builtin_amdgcn_readlane(x, 48);
+    return (a + b) + (c + d);
+}
+
+__device__ __forceinline__ unsigned wave_sum_u32(unsigned x) {
+    // counts are < 2^24 per wave-step, exact in the float pipeline
+    return (unsigned)wave_sum((float)x);
+}
+
+// ---------------------------------------------------------------------------------------
+// Element traits: X = elements per 16-byte chunk.
+template <typename T> struct Elem;
+template <> struct Elem<uint16_t> { static constexpr int X = 8; };
+template <> struct Elem<float>    { static constexpr int X = 4; };
+
+__device__ __forceinline__ uint4 ld16(const void* p) {
+    return *reinterpret_cast<const uint4*>(p);
+}
+__device__ __forceinline__ void st16(void* p, const uint4& v) {
+    *reinterpret_cast<uint4*>(p) = v;
+}
+
+// acc += <a, b> over one 16-byte chunk, fp32 accumulation.
+__device__ __forceinline__ float dot_chunk(const uint4& a, const uint4& b, float acc, uint16_t) {
+    const half2_t* x = reinterpret_cast<const half2_t*>(&a);
+    const half2_t* y = reinterpret_cast<const half2_t*>(&b);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) acc = __builtin_amdgcn_fdot2(x[i], y[i], acc, false);
+    return acc;
+}
+__device__ __forceinline__ float dot_chunk(const uint4& a, const uint4& b, float acc, float) {
+    const float* x = reinterpret_cast<const float*>(&a);
+    const float* y = reinterpret_cast<const float*>(&b);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) acc = fmaf(x[i], y[i], acc);
+    return acc;
+}
+
+// acc[0..X) += p * chunk, fp32 accumulation.
+__device__ __forceinline__ void fma_chunk(float (&acc)[8], float p, const uint4& v, uint16_t) {
+    const _Float16* h = reinterpret_cast<const _Float16*>(&v);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) acc[i] = fmaf(p, (float)h[i], acc[i]);
+}
+__device__ __forceinline__ void fma_chunk(float (&acc)[4], float p, const uint4& v, float) {
+    const float* f = reinterpret_cast<const float*>(&v);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) acc[i] = fmaf(p, f[i], acc[i]);
+}
+
+// Final store of one output element.
+__device__ __forceinline__ void store_out(uint16_t* out, int idx, float v) {
+    const _Float16 h = (_Float16)v;  // round-to-nearest-even
+    out[idx] = __builtin_bit_cast(uint16_t, h);
+}
+__device__ __forceinline__ void store_out(float* out, int idx, float v) { out[idx] = v; }
+
+// ---------------------------------------------------------------------------------------
+// The reference's pruning predicate.
+//   fp32: leq(a, b) = a <= b.
+//   fp16: leq(uint16_t a, uint16_t b) = __hle(__half(a), __half(b)), where __half(ushort)
+//         converts the integer VALUE of the bit pattern with round-to-nearest-even, so the
+//         comparison is between the two bit patterns rounded to 11 significant bits.
+// round_prob returns the probability as the kernels will use it (rounded to T); its
+// companion `key` is the quantity the predicate compares.
+__device__ __forceinline__ float round_prob(float x, uint16_t, float* key) {
+    const _Float16 h = (_Float16)x;
+    const uint16_t bits = __builtin_bit_cast(uint16_t, h);
+    *key = (float)(_Float16)(float)bits;  // numeric value of the pattern, rounded to fp16
+    return (float)h;
+}
+__device__ __forceinline__ float round_prob(float x, float, float* key) {
+    *key = x;
+    return x;
+}
+
+}  // namespace ffa

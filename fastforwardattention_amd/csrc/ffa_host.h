@@ -1,0 +1,80 @@
+// Host-side declarations shared by the C ABI (ffa_api.cpp, pure host C++), the planner
+// and the kernel launchers (ffa_kernels.hip).
+#pragma once
+
+#include <stddef.h>
+#include <stdint.h>
+
+#include "ffa_c_api.h"
+
+namespace ffa {
+
+constexpr int kTileKeys = 64;            // keys per wave tile (= wavefront size)
+constexpr int kMaxSplits = 128;          // upper bound on workgroups per (batch, head)
+constexpr int kMaxSplitWorkgroups = 16384;  // upper bound on workgroups of a split launch
+constexpr int kMaxDynamicLdsBytes = 160 * 1024 - 4096;  // gfx950: 160 KiB LDS per CU, minus statics
+
+// Arguments of one decode step, after validation.
+struct DecodeArgs {
+    int precision;
+    int B, H, Dh, Lmax, t;
+    float scale, p;
+    const void *q, *k, *v;
+    void *k_cache, *v_cache, *out;
+    const int* seq_lengths;
+    int right_or_no_padding;
+    uint32_t* kept_count;
+    uint8_t* skip_mask;
+    void* stream;
+};
+
+// Carved-up workspace for a given plan.
+struct WorkspaceView {
+    unsigned int* cnt;  // [B*H] arrival counters, zero between launches
+    float* ml;          // [B*H, n_splits, 2]
+    float* acc;         // [B*H, n_splits, Dh]
+};
+
+inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
+
+inline int num_tiles(int t) { return t / kTileKeys + 1; }  // keys 0..t inclusive
+
+// Dynamic LDS of the one-workgroup-per-(b,h) kernel: the larger of the score buffer and
+// the cross-wave merge buffer.
+inline size_t wg_dynamic_lds_bytes(int t, int waves, int elem_bytes) {
+    const size_t scores = (size_t)num_tiles(t) * kTileKeys * sizeof(float);
+    const size_t merge = (size_t)waves * 64 * (16 / elem_bytes) * sizeof(float);
+    return scores > merge ? scores : merge;
+}
+
+// Largest n_splits any plan may carry for this problem.
+inline int max_splits_for(int bh, int max_seq_len) {
+    int by_len = (max_seq_len + kTileKeys - 1) / kTileKeys;
+    int by_grid = kMaxSplitWorkgroups / (bh > 0 ? bh : 1);
+    int m = kMaxSplits;
+    if (by_len < m) m = by_len;
+    if (by_grid < m) m = by_grid;
+    return m < 1 ? 1 : m;
+}
+
+inline size_t workspace_counter_bytes(int bh) { return align_up((size_t)bh * sizeof(unsigned int), 256); }
+
+inline size_t workspace_bytes_for(int bh, int head_dim, int n_splits) {
+    if (n_splits <= 1) return workspace_counter_bytes(bh);
+    return workspace_counter_bytes(bh) + align_up((size_t)bh * n_splits * 2 * sizeof(float), 256) +
+           (size_t)bh * n_splits * head_dim * sizeof(float);
+}
+
+// planner (ffa_plan.cpp)
+int plan_launch(int precision, int B, int H, int Dh, int t, float p, int use_default, int cus,
+                ffa_launch_plan* plan);
+int validate_plan(const ffa_launch_plan& plan, int precision, int t, float p);
+
+// launchers (ffa_kernels.hip)
+int launch_decode(const DecodeArgs& a, const ffa_launch_plan& plan, const WorkspaceView& ws);
+int launch_init_cache(int precision, void* k_dst, void* v_dst, const void* k_src,
+                      const void* v_src, int B, int H, int L, int Lmax, int Dh, void* stream);
+int launch_fill_u32(unsigned int* p, size_t n, unsigned int v, void* stream);
+int query_compute_units();
+
+}  // namespace ffa

@@ -1,0 +1,629 @@
+// gfx950 (MI355X, wave64) kernels for the FastForwardAttention decode step and the C ABI
+// declared in include/ffa_c_api.h.
+//
+// Data layout in HBM (fixed by the reference, attention.cu:1556-1609):
+//   k_cache [B,H,Dh/x,Lmax,x], x = 16/sizeof(T): for one (b,h) and one 16-byte chunk c of
+//     the head dimension, the keys are consecutive 16-byte records.  A wavefront whose
+//     lane l owns key (tile*64 + l) therefore reads 64 x 16 B = 1 KiB contiguous per
+//     load instruction, and a key's whole dot product stays inside one lane.
+//   v_cache [B,H,Lmax,Dh]: a row is Dh*sizeof(T) bytes = LPR 16-byte chunks.  Lane l owns
+//     chunk (l % LPR) of row (l / LPR) of each group of RPI = 64/LPR consecutive rows, so
+//     a load instruction again covers 1 KiB contiguous.
+// A 64-key tile is NCH = Dh/x load instructions for K and NCH for V.  The probabilities
+// computed in the K mapping (one key per lane) reach the V mapping (one row per LPR lanes)
+// through a 256-byte LDS stage per wave.
+//
+// Two decode kernels:
+//   ffa_decode_split_kernel  p == 0.  Grid (b,h,split); every wave walks 64-key tiles with
+//     an online softmax, the waves of a workgroup merge (m, l, acc) in LDS, workgroups
+//     write partials and the last one to arrive (device-scope counter) merges them.
+//   ffa_decode_wg_kernel     any p.  One workgroup per (b,h), all scores staged in LDS so
+//     that the global max and sum exist before any V row is touched, which the pruning
+//     rule needs (threshold = p * inv_sum, attention.cu:1184-1191).
+#include <hip/hip_runtime.h>
+#include <math.h>
+#include <stdint.h>
+
+#include "ffa_c_api.h"
+#include "ffa_device.h"
+#include "ffa_host.h"
+
+namespace ffa {
+
+struct DecodeParams {
+    const void* q;
+    const void* k;
+    const void* v;
+    void* k_cache;
+    void* v_cache;
+    void* out;
+    const int* seq_lengths;
+    float* ws_acc;         // [BH, n_splits, Dh]
+    float* ws_ml;          // [BH, n_splits, 2]
+    unsigned int* ws_cnt;  // [BH]
+    unsigned int* kept_count;
+    unsigned char* skip_mask;
+    int B, H, Lmax, t;
+    float scale_log2e;  // softmax_scale * log2(e): scores live in the exp2 domain
+    float p;
+    int right_or_no_padding;
+    int n_splits, tiles_per_split;
+    int bh_total;
+};
+
+// Per-(b) bounds, attention.cu:805-817.  tlen = slot of the new token = number of cached
+// keys; first = first unmasked key.  Values are clamped so that a bad seq_lengths entry
+// can never produce an out-of-bounds access.
+__device__ __forceinline__ void step_bounds(const DecodeParams& P, int b, int& tlen, int& first) {
+    tlen = P.t;
+    first = 0;
+    if (P.seq_lengths != nullptr) {
+        const int sl = P.seq_lengths[b];
+        if (P.right_or_no_padding) tlen = min(max(sl, 0), P.t);
+        else first = max(sl, 0);
+    }
+}
+
+// Append k_new, v_new at slot tlen of the (b,h) caches (attention.cu:901-914, :1246).
+// One wave: lanes < NCH move one 16-byte chunk of K and one of V each.
+template <int NCH>
+__device__ __forceinline__ void append_new_token(char* kc_bh, char* vc_bh, const char* knew,
+                                                 const char* vnew, int tlen, int Lmax, int lane) {
+    for (int c = lane; c < NCH; c += kWave) {
+        st16(kc_bh + ((size_t)c * Lmax + tlen) * 16, ld16(knew + c * 16));
+        st16(vc_bh + ((size_t)tlen * NCH + c) * 16, ld16(vnew + c * 16));
+    }
+}
+
+// ---------------------------------------------------------------------------------------
+// One 64-key tile of q.K^T for the calling wave.  Lane l owns key tile*64+l; keys beyond
+// tlen read the new token's k (valid memory) and are masked by the caller.
+// Returns the raw dot product (not yet scaled).
+template <typename T, int NCH, bool Q_LDS>
+__device__ __forceinline__ float tile_qk(const char* kc_bh, const char* knew, int key, int tlen,
+                                         int Lmax, const uint4* q_reg, const uint4* q_lds) {
+    const bool cached = key < tlen;
+    const char* kp = cached ? kc_bh + (size_t)key * 16 : knew;
+    const size_t kstr = cached ? (size_t)Lmax * 16 : 16;
+    constexpr int CG = NCH < 8 ? NCH : 8;
+    float s = 0.f;
+#pragma unroll 2
+    for (int g = 0; g < NCH / CG; ++g) {
+        uint4 kv[CG];
+#pragma unroll
+        for (int c = 0; c < CG; ++c) kv[c] = ld16(kp + (size_t)(g * CG + c) * kstr);
+#pragma unroll
+        for (int c = 0; c < CG; ++c) {
+            uint4 qc;
+            if constexpr (Q_LDS) qc = q_lds[g * CG + c];
+            else qc = q_reg[g * CG + c];
+            s = dot_chunk(kv[c], qc, s, T{});
+        }
+    }
+    return s;
+}
+
+template <typename T, int DH>
+struct Geo {
+    static constexpr int X = Elem<T>::X;      // elements per 16 B
+    static constexpr int NCH = DH / X;        // 16-byte chunks per key / per V row
+    static constexpr int LPR = NCH;           // lanes per V row
+    static constexpr int RPI = kWave / LPR;   // V rows per load instruction
+    static constexpr bool Q_LDS = NCH > 16;   // q kept in LDS when it would not fit SGPR/VGPRs
+    static constexpr int QREG = Q_LDS ? 1 : NCH;
+    static_assert(NCH >= 1 && NCH <= kWave && kWave % NCH == 0, "unsupported head dim");
+};
+
+// LDS slot of key k's probability inside a wave's 64-float stage: the V mapping reads, for
+// row group rg = lane/LPR, the NCH consecutive floats [rg*NCH, rg*NCH+NCH) = keys j*RPI+rg.
+template <int NCH, int RPI>
+__device__ __forceinline__ int stage_slot(int k) { return (k % RPI) * NCH + k / RPI; }
+
+// ---------------------------------------------------------------------------------------
+// Sequence-split exact decode (p == 0).
+template <typename T, int DH, int NW>
+__global__ void __launch_bounds__(NW * 64) ffa_decode_split_kernel(const DecodeParams P) {
+    using G = Geo<T, DH>;
+    constexpr int X = G::X, NCH = G::NCH, LPR = G::LPR, RPI = G::RPI;
+    constexpr int VG = NCH < 8 ? NCH : 8;  // V loads kept in flight per group
+
+    __shared__ float s_p[NW][kWave];
+    __shared__ float s_acc[NW][kWave * X];
+    __shared__ float s_m[NW], s_l[NW];
+    __shared__ uint4 s_q[G::Q_LDS ? NCH : 1];
+    __shared__ int s_last;
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+
+    // Workgroups are handed to the 8 XCDs round-robin by index; keep every split of one
+    // (b,h) on one XCD so that partials are merged out of the L2 they were written to.
+    const int xcd = blockIdx.x & 7, r = blockIdx.x >> 3;
+    const int split = r % P.n_splits;
+    const int bh = (r / P.n_splits) * 8 + xcd;
+    if (bh >= P.bh_total) return;
+    const int b = bh / P.H;
+
+    int tlen, first;
+    step_bounds(P, b, tlen, first);
+
+    const size_t head_bytes = (size_t)P.Lmax * DH * sizeof(T);
+    char* kc_bh = reinterpret_cast<char*>(P.k_cache) + (size_t)bh * head_bytes;
+    char* vc_bh = reinterpret_cast<char*>(P.v_cache) + (size_t)bh * head_bytes;
+    const char* knew = reinterpret_cast<const char*>(P.k) + (size_t)bh * DH * sizeof(T);
+    const char* vnew = reinterpret_cast<const char*>(P.v) + (size_t)bh * DH * sizeof(T);
+    const uint4* qg = reinterpret_cast<const uint4*>(reinterpret_cast<const char*>(P.q) +
+                                                     (size_t)bh * DH * sizeof(T));
+
+    uint4 q_reg[G::QREG];
+    if constexpr (G::Q_LDS) {
+        if (tid < NCH) s_q[tid] = qg[tid];
+        __syncthreads();
+    } else {
+#pragma unroll
+        for (int c = 0; c < NCH; ++c) q_reg[c] = qg[c];
+    }
+
+    const int ntiles = tlen / kWave + 1;  // keys 0..tlen
+    const int tile_lo = max(split * P.tiles_per_split, first / kWave);
+    const int tile_hi = min(ntiles, (split + 1) * P.tiles_per_split);
+
+    // The workgroup owning the tile of slot tlen appends the new token.  Nobody reads
+    // slot tlen from the caches in this launch (it is always taken from k, v).
+    if (wave == 0 && split == min((ntiles - 1) / P.tiles_per_split, P.n_splits - 1))
+        append_new_token<NCH>(kc_bh, vc_bh, knew, vnew, tlen, P.Lmax, lane);
+
+    const int rg = lane / LPR, dch = lane % LPR;
+    float m_run = -INFINITY, l_run = 0.f;
+    float acc[X];
+#pragma unroll
+    for (int e = 0; e < X; ++e) acc[e] = 0.f;
+
+    // V rows of load group g for this lane: rows tile*64 + (g*VG+j)*RPI + rg, j < VG.
+    auto load_v_group = [&](uint4 (&vv)[VG], int tile, int g) {
+#pragma unroll
+        for (int j = 0; j < VG; ++j) {
+            const int row = min(tile * kWave + (g * VG + j) * RPI + rg, tlen);
+            const char* vp = row < tlen ? vc_bh + ((size_t)row * NCH + dch) * 16 : vnew + dch * 16;
+            vv[j] = ld16(vp);
+        }
+    };
+
+    for (int tile = tile_lo + wave; tile < tile_hi; tile += NW) {
+        const int key = tile * kWave + lane;
+        float s = tile_qk<T, NCH, G::Q_LDS>(kc_bh, knew, key, tlen, P.Lmax, q_reg, s_q);
+        // The V loads do not depend on the scores: put the first group in flight now.
+        uint4 vv[VG];
+        load_v_group(vv, tile, 0);
+
+        const bool valid = key <= tlen && key >= first;
+        s = valid ? s * P.scale_log2e : -INFINITY;
+
+        const float m_new = fmaxf(m_run, wave_max(s));
+        // m_new == -inf only while every key seen so far is masked: acc, l are still 0.
+        const float alpha = (m_new == -INFINITY) ? 1.f : __builtin_amdgcn_exp2f(m_run - m_new);
+        const float pr = valid ? __builtin_amdgcn_exp2f(s - m_new) : 0.f;
+        l_run = l_run * alpha + pr;
+        m_run = m_new;
+
+        __builtin_amdgcn_wave_barrier();
+        s_p[wave][stage_slot<NCH, RPI>(lane)] = pr;
+        __builtin_amdgcn_wave_barrier();
+
+#pragma unroll
+        for (int e = 0; e < X; ++e) acc[e] *= alpha;
+
+        const float* pst = &s_p[wave][rg * NCH];
+#pragma unroll
+        for (int g = 0; g < NCH / VG; ++g) {
+            uint4 vn[VG];
+            if (g + 1 < NCH / VG) load_v_group(vn, tile, g + 1);
+#pragma unroll
+            for (int j = 0; j < VG; ++j) fma_chunk(acc, pst[g * VG + j], vv[j], T{});
+            if (g + 1 < NCH / VG) {
+#pragma unroll
+                for (int j = 0; j < VG; ++j) vv[j] = vn[j];
+            }
+        }
+        __builtin_amdgcn_wave_barrier();
+    }
+
+    // ---- merge the waves of this workgroup (LDS) ----
+    l_run = wave_sum(l_run);
+    if (lane == 0) { s_m[wave] = m_run; s_l[wave] = l_run; }
+#pragma unroll
+    for (int e = 0; e < X; ++e) s_acc[wave][lane * X + e] = acc[e];
+    __syncthreads();
+
+    float M = -INFINITY;
+#pragma unroll
+    for (int w = 0; w < NW; ++w) M = fmaxf(M, s_m[w]);
+    float L = 0.f;
+    float wgt[NW];
+#pragma unroll
+    for (int w = 0; w < NW; ++w) {
+        wgt[w] = (s_m[w] == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(s_m[w] - M);
+        L += wgt[w] * s_l[w];
+    }
+
+    T* out = reinterpret_cast<T*>(P.out) + (size_t)bh * DH;
+    float* wa = P.ws_acc + ((size_t)bh * P.n_splits + split) * DH;
+    for (int d = tid; d < DH; d += NW * 64) {
+        float o = 0.f;
+#pragma unroll
+        for (int w = 0; w < NW; ++w) {
+            float ow = 0.f;
+#pragma unroll
+            for (int g = 0; g < RPI; ++g) ow += s_acc[w][g * DH + d];
+            o += wgt[w] * ow;
+        }
+        if (P.n_splits == 1) store_out(out, d, L > 0.f ? o / L : 0.f);
+        else wa[d] = o;
+    }
+    if (P.n_splits == 1) return;
+
+    // ---- publish the partial; the last workgroup to arrive merges all splits ----
+    if (tid == 0) {
+        float* ml = P.ws_ml + ((size_t)bh * P.n_splits + split) * 2;
+        ml[0] = M;
+        ml[1] = L;
+    }
+    __threadfence();
+    __syncthreads();
+    if (tid == 0) {
+        const unsigned prev = atomicAdd(&P.ws_cnt[bh], 1u);
+        s_last = (prev == (unsigned)(P.n_splits - 1));
+    }
+    __syncthreads();
+    if (!s_last) return;
+    __threadfence();
+
+    const float* ml = P.ws_ml + (size_t)bh * P.n_splits * 2;
+    float Mg = -INFINITY;
+    for (int s = 0; s < P.n_splits; ++s) Mg = fmaxf(Mg, __builtin_nontemporal_load(&ml[2 * s]));
+    for (int d = tid; d < DH; d += NW * 64) {
+        float o = 0.f, Lg = 0.f;
+        for (int s = 0; s < P.n_splits; ++s) {
+            const float ms = __builtin_nontemporal_load(&ml[2 * s]);
+            const float w = (ms == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(ms - Mg);
+            Lg += w * __builtin_nontemporal_load(&ml[2 * s + 1]);
+            o += w * __builtin_nontemporal_load(&P.ws_acc[((size_t)bh * P.n_splits + s) * DH + d]);
+        }
+        store_out(out, d, Lg > 0.f ? o / Lg : 0.f);
+    }
+    if (tid == 0) P.ws_cnt[bh] = 0u;  // ready for the next launch on this stream
+}
+
+// ---------------------------------------------------------------------------------------
+// One workgroup per (b,h): exact (p == 0) or pruned (p > 0) decode with LDS-staged scores.
+// Dynamic LDS: max(ntiles*64 scores, NW*64*X merge floats) * 4 bytes.
+template <typename T, int DH, int NW>
+__global__ void __launch_bounds__(NW * 64) ffa_decode_wg_kernel(const DecodeParams P) {
+    using G = Geo<T, DH>;
+    constexpr int X = G::X, NCH = G::NCH, LPR = G::LPR, RPI = G::RPI;
+    constexpr int VG = NCH < 8 ? NCH : 8;
+    constexpr int NT = NW * 64;
+
+    extern __shared__ float s_dyn[];
+    float* s_sc = s_dyn;
+    __shared__ float s_red[NW];
+    __shared__ unsigned s_cnt[NW];
+    __shared__ uint4 s_q[G::Q_LDS ? NCH : 1];
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int bh = blockIdx.x;
+    const int b = bh / P.H;
+
+    int tlen, first;
+    step_bounds(P, b, tlen, first);
+
+    const size_t head_bytes = (size_t)P.Lmax * DH * sizeof(T);
+    char* kc_bh = reinterpret_cast<char*>(P.k_cache) + (size_t)bh * head_bytes;
+    char* vc_bh = reinterpret_cast<char*>(P.v_cache) + (size_t)bh * head_bytes;
+    const char* knew = reinterpret_cast<const char*>(P.k) + (size_t)bh * DH * sizeof(T);
+    const char* vnew = reinterpret_cast<const char*>(P.v) + (size_t)bh * DH * sizeof(T);
+    const uint4* qg = reinterpret_cast<const uint4*>(reinterpret_cast<const char*>(P.q) +
+                                                     (size_t)bh * DH * sizeof(T));
+
+    uint4 q_reg[G::QREG];
+    if constexpr (G::Q_LDS) {
+        if (tid < NCH) s_q[tid] = qg[tid];
+        __syncthreads();
+    } else {
+#pragma unroll
+        for (int c = 0; c < NCH; ++c) q_reg[c] = qg[c];
+    }
+
+    const int ntiles = tlen / kWave + 1;
+    const int tile_lo = min(first / kWave, ntiles);  // tiles below are fully masked
+    const bool pruned = P.p > 0.f;
+
+    if (wave == 0) append_new_token<NCH>(kc_bh, vc_bh, knew, vnew, tlen, P.Lmax, lane);
+
+    // ---- phase 1: scores (exp2 domain) to LDS, running max ----
+    float mx = -INFINITY;
+    for (int tile = tile_lo + wave; tile < ntiles; tile += NW) {
+        const int key = tile * kWave + lane;
+        float s = tile_qk<T, NCH, G::Q_LDS>(kc_bh, knew, key, tlen, P.Lmax, q_reg, s_q);
+        const bool valid = key <= tlen && key >= first;
+        s = valid ? s * P.scale_log2e : -INFINITY;
+        s_sc[key] = s;
+        mx = fmaxf(mx, s);
+    }
+    mx = wave_max(mx);
+    if (lane == 0) s_red[wave] = mx;
+    __syncthreads();
+    float M = -INFINITY;
+#pragma unroll
+    for (int w = 0; w < NW; ++w) M = fmaxf(M, s_red[w]);
+    const bool all_masked = (M == -INFINITY);
+    if (all_masked) M = 0.f;
+    __syncthreads();  // s_red is reused below
+
+    // ---- phase 2: e_i = exp(s_i - max), sum ----
+    float sum = 0.f;
+    for (int i = tile_lo * kWave + tid; i < ntiles * kWave; i += NT) {
+        const float e = __builtin_amdgcn_exp2f(s_sc[i] - M);  // exp2(-inf) = 0 for masked keys
+        s_sc[i] = e;
+        sum += e;
+    }
+    sum = wave_sum(sum);
+    if (lane == 0) s_red[wave] = sum;
+    __syncthreads();
+    float S = 0.f;
+#pragma unroll
+    for (int w = 0; w < NW; ++w) S += s_red[w];
+
+    // p == 0: exact softmax, the 1/S factor is applied once at the end.
+    // p  > 0: the reference's rule, to the letter (attention.cu:1122-1126, :1184-1191):
+    //         inv = 1/(S+1e-6); P_i = T(e_i*inv); thr = T(p*inv); drop i<tlen iff leq(P_i,thr).
+    float out_scale = S > 0.f ? 1.f / S : 0.f;
+    if (pruned) {
+        const float inv = 1.f / (S + 1.e-6f);
+        float thr_key;
+        (void)round_prob(P.p * inv, T{}, &thr_key);
+        unsigned kept = 0;
+        for (int i = tile_lo * kWave + tid; i < ntiles * kWave; i += NT) {
+            float key_i;
+            const float Pi = round_prob(s_sc[i] * inv, T{}, &key_i);
+            const bool in_range = i >= first && i <= tlen;
+            const bool drop = !in_range || (i < tlen && key_i <= thr_key);
+            s_sc[i] = drop ? -1.f : Pi;
+            if (i < tlen) {
+                kept += drop ? 0u : 1u;
+                if (P.skip_mask) P.skip_mask[(size_t)bh * P.Lmax + i] = drop ? 1 : 0;
+            }
+        }
+        if (P.skip_mask)  // keys of fully masked leading tiles are dropped too
+            for (int i = tid; i < min(tile_lo * kWave, tlen); i += NT)
+                P.skip_mask[(size_t)bh * P.Lmax + i] = 1;
+        if (P.kept_count) {
+            kept = wave_sum_u32(kept);
+            if (lane == 0) s_cnt[wave] = kept;
+        }
+        out_scale = 1.f;
+    } else {
+        if (P.skip_mask)
+            for (int i = tid; i < tlen; i += NT)
+                P.skip_mask[(size_t)bh * P.Lmax + i] = (i < first) ? 1 : 0;
+    }
+    __syncthreads();
+    if (P.kept_count && tid == 0) {
+        unsigned tot = 0;
+        if (pruned) {
+#pragma unroll
+            for (int w = 0; w < NW; ++w) tot += s_cnt[w];
+        } else {
+            tot = (unsigned)max(tlen - min(first, tlen), 0);
+        }
+        P.kept_count[bh] = tot;
+    }
+
+    // ---- phase 3: P.V with the skip fused in ----
+    const int rg = lane / LPR, dch = lane % LPR;
+    float acc[X];
+#pragma unroll
+    for (int e = 0; e < X; ++e) acc[e] = 0.f;
+    for (int tile = tile_lo + wave; tile < ntiles; tile += NW) {
+#pragma unroll 1
+        for (int g = 0; g < NCH / VG; ++g) {
+            uint4 vv[VG];
+            float pj[VG];
+#pragma unroll
+            for (int j = 0; j < VG; ++j) {
+                const int row = tile * kWave + (g * VG + j) * RPI + rg;
+                pj[j] = s_sc[row];
+                const bool keep = pruned ? (pj[j] >= 0.f) : (row <= tlen);
+                vv[j] = make_uint4(0, 0, 0, 0);
+                if (keep) {
+                    const char* vp = row < tlen ? vc_bh + ((size_t)row * NCH + dch) * 16 : vnew + dch * 16;
+                    vv[j] = ld16(vp);
+                } else {
+                    pj[j] = 0.f;
+                }
+            }
+#pragma unroll
+            for (int j = 0; j < VG; ++j) fma_chunk(acc, pj[j], vv[j], T{});
+        }
+    }
+
+    // ---- merge the waves (the score buffer is dead now and is reused) ----
+    __syncthreads();
+    float* s_acc = s_dyn;
+#pragma unroll
+    for (int e = 0; e < X; ++e) s_acc[(wave * kWave + lane) * X + e] = acc[e];
+    __syncthreads();
+    T* out = reinterpret_cast<T*>(P.out) + (size_t)bh * DH;
+    for (int d = tid; d < DH; d += NT) {
+        float o = 0.f;
+        for (int w = 0; w < NW; ++w)
+#pragma unroll
+            for (int g = 0; g < RPI; ++g) o += s_acc[w * kWave * X + g * DH + d];
+        store_out(out, d, all_masked ? 0.f : o * out_scale);
+    }
+}
+
+// ---------------------------------------------------------------------------------------
+// Cache construction (attention.cu:1556-1609).  One workgroup moves a tile of TK keys of
+// one (b,h): coalesced row reads [64 keys x Dh] -> LDS -> coalesced 1 KiB chunk-row writes
+// for K; V is a straight strided copy.
+template <int NCH, int TK>
+__global__ void __launch_bounds__(256) ffa_init_cache_kernel(uint4* __restrict__ k_dst,
+                                                             uint4* __restrict__ v_dst,
+                                                             const uint4* __restrict__ k_src,
+                                                             const uint4* __restrict__ v_src,
+                                                             int L, int Lmax) {
+    __shared__ uint4 s_tile[NCH * (TK + 1)];  // [chunk][key], one chunk of padding per row
+    const int bh = blockIdx.y;
+    const int l0 = blockIdx.x * TK;
+    const int nkeys = min(TK, L - l0);
+    const uint4* ks = k_src + ((size_t)bh * L + l0) * NCH;
+    const uint4* vs = v_src + ((size_t)bh * L + l0) * NCH;
+    uint4* kd = k_dst + (size_t)bh * Lmax * NCH;
+    uint4* vd = v_dst + ((size_t)bh * Lmax + l0) * NCH;
+    // V: contiguous copy of nkeys*NCH chunks.
+    for (int i = threadIdx.x; i < nkeys * NCH; i += 256) vd[i] = vs[i];
+    // K: read [key][chunk] (contiguous), write [chunk][key].
+    for (int i = threadIdx.x; i < nkeys * NCH; i += 256) {
+        const int key = i / NCH, c = i % NCH;
+        s_tile[c * (TK + 1) + key] = ks[i];
+    }
+    __syncthreads();
+    for (int i = threadIdx.x; i < TK * NCH; i += 256) {
+        const int c = i / TK, key = i % TK;
+        if (key < nkeys) kd[(size_t)c * Lmax + l0 + key] = s_tile[c * (TK + 1) + key];
+    }
+}
+
+__global__ void ffa_fill_u32_kernel(unsigned int* p, size_t n, unsigned int v) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) p[i] = v;
+}
+
+// ---------------------------------------------------------------------------------------
+// Host-side dispatch.
+static int check_launch() {
+    return hipGetLastError() == hipSuccess ? FFA_OK : FFA_ERR_LAUNCH;
+}
+
+template <typename T, int DH, int NW>
+static int launch_split(const DecodeParams& P, hipStream_t st) {
+    const int groups = (P.bh_total + 7) / 8;
+    const dim3 grid((unsigned)(groups * 8 * P.n_splits));
+    hipLaunchKernelGGL((ffa_decode_split_kernel<T, DH, NW>), grid, dim3(NW * 64), 0, st, P);
+    return check_launch();
+}
+
+template <typename T, int DH, int NW>
+static int launch_wg(const DecodeParams& P, size_t lds_bytes, hipStream_t st) {
+    auto kern = ffa_decode_wg_kernel<T, DH, NW>;
+    if (lds_bytes > 48 * 1024) {
+        // Raise the dynamic-LDS ceiling once per instantiation (gfx950: 160 KiB per CU).
+        static int raised = 0;
+        if (!raised) {
+            if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                    hipFuncAttributeMaxDynamicSharedMemorySize,
+                                    kMaxDynamicLdsBytes) != hipSuccess) {
+                (void)hipGetLastError();
+                return FFA_ERR_LAUNCH;
+            }
+            raised = 1;
+        }
+    }
+    hipLaunchKernelGGL(kern, dim3((unsigned)P.bh_total), dim3(NW * 64), lds_bytes, st, P);
+    return check_launch();
+}
+
+template <typename T, int DH>
+static int dispatch_waves(const DecodeParams& P, const ffa_launch_plan& plan, hipStream_t st) {
+    if (plan.kind == FFA_LAUNCH_SPLIT) {
+        switch (plan.waves_per_wg) {
+            case 1: return launch_split<T, DH, 1>(P, st);
+            case 2: return launch_split<T, DH, 2>(P, st);
+            case 4: return launch_split<T, DH, 4>(P, st);
+            case 8: return launch_split<T, DH, 8>(P, st);
+            default: return FFA_ERR_PLAN;
+        }
+    }
+    const size_t lds = wg_dynamic_lds_bytes(P.t, plan.waves_per_wg, (int)sizeof(T));
+    switch (plan.waves_per_wg) {
+        case 1: return launch_wg<T, DH, 1>(P, lds, st);
+        case 2: return launch_wg<T, DH, 2>(P, lds, st);
+        case 4: return launch_wg<T, DH, 4>(P, lds, st);
+        case 8: return launch_wg<T, DH, 8>(P, lds, st);
+        case 16: return launch_wg<T, DH, 16>(P, lds, st);
+        default: return FFA_ERR_PLAN;
+    }
+}
+
+template <typename T>
+static int dispatch_head_dim(const DecodeParams& P, int head_dim, const ffa_launch_plan& plan,
+                             hipStream_t st) {
+    switch (head_dim) {
+        case 64: return dispatch_waves<T, 64>(P, plan, st);
+        case 128: return dispatch_waves<T, 128>(P, plan, st);
+        case 256: return dispatch_waves<T, 256>(P, plan, st);
+        default: return FFA_ERR_HEAD_DIM;
+    }
+}
+
+int launch_decode(const DecodeArgs& a, const ffa_launch_plan& plan, const WorkspaceView& ws) {
+    DecodeParams P;
+    P.q = a.q; P.k = a.k; P.v = a.v;
+    P.k_cache = a.k_cache; P.v_cache = a.v_cache; P.out = a.out;
+    P.seq_lengths = a.seq_lengths;
+    P.ws_acc = ws.acc; P.ws_ml = ws.ml; P.ws_cnt = ws.cnt;
+    P.kept_count = a.kept_count; P.skip_mask = a.skip_mask;
+    P.B = a.B; P.H = a.H; P.Lmax = a.Lmax; P.t = a.t;
+    P.scale_log2e = a.scale * kLog2e;
+    P.p = a.p;
+    P.right_or_no_padding = a.right_or_no_padding;
+    P.n_splits = plan.n_splits; P.tiles_per_split = plan.tiles_per_split;
+    P.bh_total = a.B * a.H;
+    hipStream_t st = reinterpret_cast<hipStream_t>(a.stream);
+    if (a.precision == FFA_PRECISION_F16) return dispatch_head_dim<uint16_t>(P, a.Dh, plan, st);
+    return dispatch_head_dim<float>(P, a.Dh, plan, st);
+}
+
+int launch_init_cache(int precision, void* k_dst, void* v_dst, const void* k_src,
+                      const void* v_src, int B, int H, int L, int Lmax, int Dh, void* stream) {
+    const int nch = Dh * (precision / 8) / 16;
+    const int tk = nch <= 32 ? 64 : 32;  // keeps the LDS tile under 64 KiB
+    const dim3 grid((unsigned)((L + tk - 1) / tk), (unsigned)(B * H));
+    hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+    auto kd = reinterpret_cast<uint4*>(k_dst);
+    auto vd = reinterpret_cast<uint4*>(v_dst);
+    auto ks = reinterpret_cast<const uint4*>(k_src);
+    auto vs = reinterpret_cast<const uint4*>(v_src);
+    switch (nch) {
+        case 8: hipLaunchKernelGGL((ffa_init_cache_kernel<8, 64>), grid, dim3(256), 0, st, kd, vd, ks, vs, L, Lmax); break;
+        case 16: hipLaunchKernelGGL((ffa_init_cache_kernel<16, 64>), grid, dim3(256), 0, st, kd, vd, ks, vs, L, Lmax); break;
+        case 32: hipLaunchKernelGGL((ffa_init_cache_kernel<32, 64>), grid, dim3(256), 0, st, kd, vd, ks, vs, L, Lmax); break;
+        case 64: hipLaunchKernelGGL((ffa_init_cache_kernel<64, 32>), grid, dim3(256), 0, st, kd, vd, ks, vs, L, Lmax); break;
+        default: return FFA_ERR_HEAD_DIM;
+    }
+    return check_launch();
+}
+
+int launch_fill_u32(unsigned int* p, size_t n, unsigned int v, void* stream) {
+    if (n == 0) return FFA_OK;
+    const unsigned blocks = (unsigned)((n + 255) / 256);
+    hipLaunchKernelGGL(ffa_fill_u32_kernel, dim3(blocks), dim3(256), 0,
+                       reinterpret_cast<hipStream_t>(stream), p, n, v);
+    return check_launch();
+}
+
+int query_compute_units() {
+    static int cached = 0;  // one device model per process
+    if (cached > 0) return cached;
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) { (void)hipGetLastError(); return -1; }
+    int cus = 0;
+    if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) {
+        (void)hipGetLastError();
+        return -1;
+    }
+    cached = cus;
+    return cus;
+}
+
+}  // namespace ffa

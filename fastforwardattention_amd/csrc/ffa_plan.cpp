@@ -1,0 +1,109 @@
+// Launch planner for the gfx950 decode kernels.  Pure host code, no HIP calls.
+//
+// Stands where the reference has get_launch_params (kernel_launch_utils.h:135-180), which
+// searches threads-per-block x threads-per-key x threads-per-value with a fitted time
+// model.  On a 256-CU wave64 part with the reference's K layout the per-key work is best
+// kept in one lane (threads_per_key = 1: every load instruction is 1 KiB contiguous), so
+// the quantities that matter are how many wavefronts share a (batch, head) and how the
+// sequence is split across workgroups.
+#include <math.h>
+
+#include "ffa_host.h"
+
+namespace ffa {
+
+static int pow2_floor(int v) {
+    int p = 1;
+    while (p * 2 <= v) p *= 2;
+    return p;
+}
+
+static int ceil_div(int a, int b) { return (a + b - 1) / b; }
+
+static void fill(ffa_launch_plan* plan, int kind, int waves, int n_splits, int tiles_per_split) {
+    plan->kind = kind;
+    plan->waves_per_wg = waves;
+    plan->threads_per_key = 1;
+    plan->keys_per_wave = kTileKeys;
+    plan->n_splits = n_splits;
+    plan->tiles_per_split = tiles_per_split;
+    plan->reserved[0] = plan->reserved[1] = 0;
+}
+
+// Largest power-of-two wave count (<= 16) whose score buffer + merge buffer fit in LDS and
+// that still leaves every wave at least one tile.
+static int wg_waves_for(int ntiles, int want) {
+    int w = pow2_floor(want < 1 ? 1 : want);
+    if (w > 16) w = 16;
+    while (w > 1 && w > ntiles) w /= 2;
+    return w;
+}
+
+int plan_launch(int precision, int B, int H, int Dh, int t, float p, int use_default, int cus,
+                ffa_launch_plan* plan) {
+    if (plan == nullptr) return FFA_ERR_NULL_POINTER;
+    if (precision != FFA_PRECISION_F16 && precision != FFA_PRECISION_F32) return FFA_ERR_DTYPE;
+    if (Dh != 64 && Dh != 128 && Dh != 256) return FFA_ERR_HEAD_DIM;
+    if (B <= 0 || H <= 0) return FFA_ERR_SHAPE;
+    if (t < 0) return FFA_ERR_TIMESTEP;
+    if (!(p >= 0.f)) return FFA_ERR_PROB_THRESH;
+    if (cus <= 0) cus = 256;
+
+    const int ntiles = num_tiles(t);
+    const int bh = B * H;
+    const bool fits_wg = wg_dynamic_lds_bytes(t, 16, precision / 8) <= (size_t)kMaxDynamicLdsBytes;
+
+    if (use_default) {
+        // One workgroup per (batch, head); workgroup size by sequence length like the
+        // FasterTransformer table (kernel_launch_utils.h:147-154: 64 / 128 / 256 threads).
+        if (!fits_wg) return FFA_ERR_TOO_LONG;
+        const int waves = t < 32 ? 1 : (t < 2048 ? 2 : 4);
+        fill(plan, FFA_LAUNCH_WORKGROUP, wg_waves_for(ntiles, waves), 1, ntiles);
+        return FFA_OK;
+    }
+
+    if (p > 0.f) {
+        // Pruning needs the global max and sum before V: one workgroup per (b,h), as many
+        // waves as there are tiles to keep in flight (up to 16).
+        if (!fits_wg) return FFA_ERR_TOO_LONG;
+        fill(plan, FFA_LAUNCH_WORKGROUP, wg_waves_for(ntiles, ceil_div(ntiles, 4)), 1, ntiles);
+        return FFA_OK;
+    }
+
+    // Exact path: split the sequence so that the launch has about `target` workgroups.
+    const int waves = wg_waves_for(ntiles, 4);
+    const int target = 6 * cus;
+    int n_splits = target / bh;
+    const int cap = max_splits_for(bh, (t + 1));
+    if (n_splits > cap) n_splits = cap;
+    if (n_splits > ceil_div(ntiles, waves)) n_splits = ceil_div(ntiles, waves);
+    if (n_splits < 1) n_splits = 1;
+    const int tps = ceil_div(ntiles, n_splits);
+    n_splits = ceil_div(ntiles, tps);
+    fill(plan, FFA_LAUNCH_SPLIT, waves, n_splits, tps);
+    return FFA_OK;
+}
+
+int validate_plan(const ffa_launch_plan& plan, int precision, int t, float p) {
+    const int w = plan.waves_per_wg;
+    if (w != 1 && w != 2 && w != 4 && w != 8 && w != 16) return FFA_ERR_PLAN;
+    if (plan.threads_per_key != 1 || plan.keys_per_wave != kTileKeys) return FFA_ERR_PLAN;
+    if (plan.n_splits < 1 || plan.n_splits > kMaxSplits || plan.tiles_per_split < 1) return FFA_ERR_PLAN;
+    const int ntiles = num_tiles(t);
+    switch (plan.kind) {
+        case FFA_LAUNCH_WORKGROUP:
+            if (plan.n_splits != 1) return FFA_ERR_PLAN;
+            if (wg_dynamic_lds_bytes(t, w, precision / 8) > (size_t)kMaxDynamicLdsBytes)
+                return FFA_ERR_TOO_LONG;
+            return FFA_OK;
+        case FFA_LAUNCH_SPLIT:
+            if (p > 0.f) return FFA_ERR_PLAN;  // the split kernel is the exact path only
+            if (w > 8) return FFA_ERR_PLAN;
+            if ((long long)plan.n_splits * plan.tiles_per_split < ntiles) return FFA_ERR_PLAN;
+            return FFA_OK;
+        default:
+            return FFA_ERR_PLAN;
+    }
+}
+
+}  // namespace ffa

@@ -1,0 +1,158 @@
+/*
+ * ffa_c_api.h -- C ABI of the MI355X (gfx950) decode-attention engine.
+ *
+ * Drop-in boundary for the decode step of szeighami/FastForwardAttention.  Every entry
+ * point names the reference interface it replaces (file:line in the reference tree).
+ * Plain C: pointers, ints and floats only; no torch types, no C++ templates.
+ *
+ * Conventions
+ *   - all data pointers are DEVICE pointers on the current HIP device, 16-byte aligned;
+ *   - fp16 is passed as uint16_t bit patterns (the reference does the same:
+ *     attention.cu:1534, torch_ffa_api.cpp:124-126);
+ *   - `stream` is a hipStream_t passed as void* (NULL = the default stream, which is
+ *     what the reference always uses: attention.cu:1504);
+ *   - the library never allocates: caches, outputs and the workspace belong to the caller;
+ *   - every function returns an ffa_status (0 = FFA_OK) and never throws, aborts or
+ *     prints.  The reference prints and continues (attention.cu:1444-1451, :1529).
+ *
+ * Layouts (fixed by the reference, attention.cu:1556-1609)
+ *   k_cache [B, H, Dh/x, Lmax, x]   x = 16 / sizeof(T)  (8 for fp16, 4 for fp32)
+ *   v_cache [B, H, Lmax, Dh]
+ *   q, k, v, out  [B, H, Dh] contiguous
+ */
+#ifndef FFA_C_API_H
+#define FFA_C_API_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define FFA_API_VERSION 1
+
+typedef enum ffa_status {
+    FFA_OK = 0,
+    FFA_ERR_NULL_POINTER = 1,   /* a required pointer is NULL                                */
+    FFA_ERR_DTYPE = 2,          /* precision is neither 16 nor 32                            */
+    FFA_ERR_HEAD_DIM = 3,       /* Dh not one of 64, 128, 256                                */
+    FFA_ERR_SHAPE = 4,          /* B, H, L or Lmax not positive, or L > Lmax                 */
+    FFA_ERR_TIMESTEP = 5,       /* t outside [0, Lmax)                                       */
+    FFA_ERR_ALIGNMENT = 6,      /* a pointer is not 16-byte aligned                          */
+    FFA_ERR_WORKSPACE = 7,      /* workspace NULL/too small for the chosen plan              */
+    FFA_ERR_PLAN = 8,           /* malformed launch plan                                     */
+    FFA_ERR_TOO_LONG = 9,       /* t+1 scores do not fit the LDS of a one-workgroup launch   */
+    FFA_ERR_PROB_THRESH = 10,   /* p is negative or NaN                                      */
+    FFA_ERR_LAUNCH = 11,        /* the HIP runtime refused the launch                        */
+    FFA_ERR_NO_DEVICE = 12      /* no usable gfx950 device / HIP runtime error               */
+} ffa_status;
+
+/* precision codes: the same integers the reference passes to get_launch_params
+ * (torch_ffa_api.cpp:174). */
+#define FFA_PRECISION_F16 16
+#define FFA_PRECISION_F32 32
+
+/* Launch kinds. */
+#define FFA_LAUNCH_WORKGROUP 0  /* one workgroup per (batch, head); scores staged in LDS;   */
+                                /* any p >= 0.  The analogue of the reference's launch.     */
+#define FFA_LAUNCH_SPLIT 1      /* sequence split over n_splits workgroups per (batch,      */
+                                /* head), online softmax, last-arriver combine; p == 0 only */
+
+/* Replaces the (tpb, tpv, tpk) triple of kernel_launch_utils.h:135-180. */
+typedef struct ffa_launch_plan {
+    int32_t kind;             /* FFA_LAUNCH_*                                              */
+    int32_t waves_per_wg;     /* wave64 wavefronts per workgroup: 1, 2, 4, 8 or 16         */
+    int32_t threads_per_key;  /* lanes cooperating on one key's q.k (1 in this version)    */
+    int32_t keys_per_wave;    /* 64 / threads_per_key                                      */
+    int32_t n_splits;         /* workgroups per (batch, head); 1 for FFA_LAUNCH_WORKGROUP  */
+    int32_t tiles_per_split;  /* 64-key tiles each split walks                             */
+    int32_t reserved[2];
+} ffa_launch_plan;
+
+int ffa_api_version(void);
+const char* ffa_status_string(int status);
+
+/* Number of compute units of the current device (256 on MI355X); <= 0 if none. */
+int ffa_device_compute_units(void);
+
+/*
+ * Launch planner.  Replaces get_launch_params (kernel_launch_utils.h:135-180).
+ *   precision  16 | 32;  t = number of cached keys at the step being planned (the
+ *   reference plans once on the prompt length, torch_ffa_api.cpp:176; this planner is
+ *   cheap enough to be called per step);  prob_thresh: the p the step will use;
+ *   use_default_kernel_launch != 0 -> one workgroup per (batch, head), workgroup size by
+ *   sequence length, like the FasterTransformer table at kernel_launch_utils.h:137-154;
+ *   == 0 -> tuned plan for `compute_units` CUs (pass 0 to query the current device).
+ */
+int ffa_plan_launch(int precision, int batch_size, int head_num, int head_dim,
+                    int t, float prob_thresh, int use_default_kernel_launch,
+                    int compute_units, ffa_launch_plan* plan);
+
+/* Bytes of device workspace sufficient for ANY plan this library produces for the
+ * given problem (split partials + arrival counters). */
+size_t ffa_workspace_bytes(int batch_size, int head_num, int head_dim, int max_seq_len);
+
+/* Zero the arrival counters of a fresh workspace (once, before first use). */
+int ffa_workspace_init(void* workspace, size_t workspace_bytes, void* stream);
+
+/*
+ * Cache construction.  Replaces invokeTranspose4dBatchMajor<T>
+ * (torch_ffa_api.cpp:14-47; attention.cu:1611-1689) -- same argument order.
+ *   k_dst [B,H,Dh/x,Lmax,x], v_dst [B,H,Lmax,Dh]  <-  k_src, v_src [B,H,L,Dh].
+ * Slots l >= seq_len are left untouched, as in the reference.
+ */
+int ffa_init_cache_f16(uint16_t* k_dst, uint16_t* v_dst, const uint16_t* k_src,
+                       const uint16_t* v_src, int batch_size, int seq_len, int max_seq_len,
+                       int head_dim, int head_num, void* stream);
+int ffa_init_cache_f32(float* k_dst, float* v_dst, const float* k_src, const float* v_src,
+                       int batch_size, int seq_len, int max_seq_len, int head_dim,
+                       int head_num, void* stream);
+
+/*
+ * One decode-attention step.  Replaces call_attention<T> (c_ffa_api.h:10-14;
+ * attention.cu:1512-1554) and do_attention<T> (c_ffa_api.h:17-20): appends k, v at
+ * cache slot t and writes out[b,h,:] = sum_i P_i V_i over keys first_key .. t.
+ *   seq_lengths (device int[B]) may be NULL.  With right_or_no_padding != 0 it is the
+ *   per-sample slot/length that replaces t (attention.cu:809-811; every entry must be
+ *   <= t); with right_or_no_padding == 0 it is the index of the first real key of a
+ *   left-padded sample (attention.cu:814-817).
+ *   prob_thresh == 0: exact attention.  prob_thresh > 0: the reference's pruning rule
+ *   (attention.cu:1184-1191): key i < t is dropped iff leq(T(e_i*inv), T(p*inv)).
+ *   plan: NULL -> planned internally as ffa_plan_launch(..., use_default = 0).
+ *   workspace: required unless the plan is FFA_LAUNCH_WORKGROUP.
+ */
+int ffa_attention_f16(int batch_size, int head_num, int head_dim, int max_seq_len,
+                      float softmax_scale, int t, const uint16_t* q, const uint16_t* k,
+                      const uint16_t* v, uint16_t* k_cache, uint16_t* v_cache, uint16_t* out,
+                      const int* seq_lengths, float prob_thresh, const ffa_launch_plan* plan,
+                      int right_or_no_padding, void* workspace, size_t workspace_bytes,
+                      void* stream);
+int ffa_attention_f32(int batch_size, int head_num, int head_dim, int max_seq_len,
+                      float softmax_scale, int t, const float* q, const float* k,
+                      const float* v, float* k_cache, float* v_cache, float* out,
+                      const int* seq_lengths, float prob_thresh, const ffa_launch_plan* plan,
+                      int right_or_no_padding, void* workspace, size_t workspace_bytes,
+                      void* stream);
+
+/*
+ * Same step with pruning diagnostics (no counterpart in the reference, which never
+ * reports what it skipped; needed to report the fraction of keys skipped):
+ *   kept_count  device uint32[B*H] or NULL: number of cached keys i < t whose V row was
+ *               read (overwritten, not accumulated);
+ *   skip_mask   device uint8[B*H*Lmax] or NULL: 1 where key i < t was dropped.
+ * Diagnostics need the one-workgroup launch: a NULL plan is planned that way, an
+ * FFA_LAUNCH_SPLIT plan is rejected with FFA_ERR_PLAN.  With prob_thresh == 0 only
+ * masked (left-padding) keys count as dropped and kept_count[b,h] = t - first_key.
+ */
+int ffa_attention_diag(int precision, int batch_size, int head_num, int head_dim,
+                       int max_seq_len, float softmax_scale, int t, const void* q,
+                       const void* k, const void* v, void* k_cache, void* v_cache, void* out,
+                       const int* seq_lengths, float prob_thresh, const ffa_launch_plan* plan,
+                       int right_or_no_padding, void* workspace, size_t workspace_bytes,
+                       uint32_t* kept_count, uint8_t* skip_mask, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* FFA_C_API_H */

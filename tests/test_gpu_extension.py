@@ -1,0 +1,120 @@
+"""GPU tests of the Python surface: class FastForwardAttn of the compiled extension
+`ff_attention`, used exactly like the reference's example (example.py:28-46)."""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from oracle.torch_attn import torch_attn_func
+
+pytestmark = pytest.mark.gpu
+
+
+def _say(*a):
+    print(*a, flush=True)
+
+
+@pytest.mark.parametrize("dtype,tol", [(torch.float16, 1e-3), (torch.float32, 1e-6)])
+@pytest.mark.parametrize("default_launch", [False, True])
+def test_example_loop(dtype, tol, default_launch):
+    """The reference demo, shrunk: B=10, H=32, Dh=64, prompt 1024 -> here prompt 200, 20 steps;
+    randn instead of rand inputs; absolute instead of relative tolerance."""
+    from ff_attention import FastForwardAttn as FFA  # the reference's import line
+    _say("example_loop", dtype, default_launch)
+    B, H, Dh, L, steps = 3, 8, 64, 200, 20
+    g = torch.Generator().manual_seed(1)
+    K = torch.randn(B, H, L, Dh, generator=g).to(dtype)
+    V = torch.randn(B, H, L, Dh, generator=g).to(dtype)
+    ffa = FFA(K.cuda(), V.cuda(), L + steps, default_launch)
+    scale = 1 / math.sqrt(Dh)
+    Kf, Vf = K.float(), V.float()
+    for i in range(steps):
+        q, k, v = (torch.randn(B, H, 1, Dh, generator=g).to(dtype) for _ in range(3))
+        t = L + i
+        out = ffa.attention(q.cuda(), k.cuda(), v.cuda(), scale, t, 0)
+        assert out.shape == (B, H, Dh) and out.dtype == dtype and out.is_cuda
+        Kf = torch.cat([Kf, k.float()], dim=-2)
+        Vf = torch.cat([Vf, v.float()], dim=-2)
+        want = torch_attn_func(q.float().view(B * H, 1, Dh), Kf.view(B * H, t + 1, Dh),
+                               Vf.view(B * H, t + 1, Dh), scale).view(B, H, Dh)
+        assert (out.float().cpu() - want).abs().max() <= tol
+
+
+def test_cache_shapes_aliasing_and_overloads():
+    from fastforwardattention_amd import FastForwardAttn as FFA
+    B, H, Dh, L, Lmax = 2, 4, 128, 70, 80
+    g = torch.Generator().manual_seed(2)
+    K = torch.randn(B, H, L, Dh, generator=g).half().cuda()
+    V = torch.randn(B, H, L, Dh, generator=g).half().cuda()
+    ffa = FFA(K, V, Lmax, False)
+    kc, vc = ffa.get_cache()
+    assert tuple(kc.shape) == (B, H, Dh // 8, Lmax, 8) and tuple(vc.shape) == (B, H, Lmax, Dh)
+    assert torch.equal(kc[:, :, :, :L, :], K.view(B, H, L, Dh // 8, 8).permute(0, 1, 3, 2, 4))
+    assert torch.equal(vc[:, :, :L], V)
+    q, k, v = (torch.randn(B, 1, H * Dh, generator=g).half().cuda() for _ in range(3))  # OPT's shape
+    o1 = ffa.attention(q, k, v, 0.1, L, 0)
+    # the caches are aliases: the append is visible through get_cache()
+    assert torch.equal(kc[:, :, :, L, :].reshape(B, H, Dh), k.view(B, H, Dh))
+    assert torch.equal(vc[:, :, L, :], v.view(B, H, Dh))
+    # 8-argument overload on the same caches: same result (slot L is rewritten with the same row)
+    o2 = ffa.attention(q, k, v, kc, vc, 0.1, L, 0)
+    assert torch.equal(o1, o2)
+    # 9-argument overload with first_key = 0 everywhere: same again
+    o3 = ffa.attention(q, k, v, kc, vc, 0.1, L, torch.zeros(B, dtype=torch.int32, device="cuda"), 0)
+    assert torch.equal(o1, o3)
+    # left padding really masks
+    sl = torch.tensor([0, 40], dtype=torch.int32, device="cuda")
+    o4 = ffa.attention(q, k, v, kc, vc, 0.1, L, sl, 0)
+    assert torch.equal(o4[0], o1[0]) and not torch.equal(o4[1], o1[1])
+    Kf = torch.cat([K, k.view(B, H, 1, Dh)], 2).float()[1, :, 40:]
+    Vf = torch.cat([V, v.view(B, H, 1, Dh)], 2).float()[1, :, 40:]
+    want = torch_attn_func(q.view(B, H, 1, Dh)[1].float(), Kf, Vf, 0.1)[:, 0]
+    assert (o4[1].float() - want).abs().max() <= 1e-3
+
+
+def test_errors_raise():
+    from fastforwardattention_amd import FastForwardAttn as FFA
+    K = torch.randn(1, 2, 10, 64).half().cuda()
+    ffa = FFA(K, K.clone(), 12, False)
+    q = torch.randn(1, 2, 64).half().cuda()
+    with pytest.raises(RuntimeError, match="timestep"):
+        ffa.attention(q, q, q, 0.1, 12, 0)           # the reference writes past the cache here
+    with pytest.raises(RuntimeError, match="elements"):
+        ffa.attention(q[:, :1], q, q, 0.1, 10, 0)
+    with pytest.raises(RuntimeError, match="dtype"):
+        ffa.attention(q.float(), q, q, 0.1, 10, 0)
+    with pytest.raises(RuntimeError, match="prob_thresh"):
+        ffa.attention(q, q, q, 0.1, 10, -1.0)
+    with pytest.raises(RuntimeError, match="head dim"):
+        FFA(torch.randn(1, 2, 10, 80).half().cuda(), torch.randn(1, 2, 10, 80).half().cuda(), 12, False)
+    with pytest.raises(RuntimeError):
+        FFA(torch.randn(1, 2, 10, 64).double().cuda(), torch.randn(1, 2, 10, 64).double().cuda(), 12, False)
+    with pytest.raises(TypeError):
+        ffa.attention(q, q, q, 0.1, 10)               # p is positional and mandatory, as in the reference
+
+
+def test_pruned_diag_and_stream():
+    from fastforwardattention_amd import FastForwardAttn as FFA
+    B, H, Dh, L = 2, 4, 64, 600
+    g = torch.Generator().manual_seed(3)
+    K = torch.randn(B, H, L, Dh, generator=g).half().cuda()
+    V = torch.randn(B, H, L, Dh, generator=g).half().cuda()
+    q, k, v = (torch.randn(B, H, Dh, generator=g).half().cuda() for _ in range(3))
+    ffa = FFA(K, V, L + 1, False)
+    exact = ffa.attention(q, k, v, 0.5, L, 0)
+    out, kept, mask = ffa.attention_diag(q, k, v, 0.5, L, 5e-2)
+    assert kept.shape == (B, H) and mask.shape == (B, H, L + 1)
+    assert torch.equal(kept.long(), L - mask[:, :, :L].sum(-1).long())
+    assert 0 < mask.float().mean() < 1
+    assert (out.float() - exact.float()).abs().max() < 0.2
+    plain = ffa.attention(q, k, v, 0.5, L, 5e-2)
+    assert torch.equal(plain, out)
+    # a side stream: the extension launches on torch's current stream
+    s = torch.cuda.Stream()
+    s.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(s):
+        o2 = ffa.attention(q, k, v, 0.5, L, 0)
+    s.synchronize()
+    assert torch.equal(o2, exact)
+    assert len(ffa.launch_plan(L, 0.0)) == 6

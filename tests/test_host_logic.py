@@ -1,0 +1,165 @@
+"""CPU tests of the host side of the C ABI: the library loads, exports every symbol that
+include/ffa_c_api.h declares, validates arguments before touching the GPU, and the launch
+planner produces consistent plans.  No kernel is launched here."""
+import ctypes as C
+import os
+import re
+
+import pytest
+
+from fastforwardattention_amd import capi
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "ffa_c_api.h")
+
+
+@pytest.fixture(scope="module")
+def lib():
+    return capi.load()
+
+
+def _declared_functions():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(ffa_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_every_declared_symbol_is_exported_and_bound(lib):
+    names = _declared_functions()
+    assert len(names) >= 11
+    for n in names:
+        assert hasattr(lib, n), f"{n} declared in ffa_c_api.h but not exported"
+    assert sorted(capi.SIGNATURES) == names, "capi.SIGNATURES out of sync with the header"
+
+
+def test_version_and_status_strings(lib):
+    assert lib.ffa_api_version() == 1
+    seen = set()
+    for code in range(0, 13):
+        s = capi.status_string(code)
+        assert s and s != "unknown status"
+        seen.add(s)
+    assert len(seen) == 13
+    assert capi.status_string(99) == "unknown status"
+
+
+def test_struct_layout_matches_header():
+    assert C.sizeof(capi.LaunchPlan) == 32
+
+
+# dummy 16-byte aligned non-null "device pointers": validation must reject the call
+# before any of them is dereferenced or a kernel is launched
+P = C.c_void_p(0x1000)
+
+
+def _attn(lib, precision=16, B=2, H=4, Dh=64, Lmax=128, scale=0.125, t=10, q=P, k=P, v=P, kc=P,
+          vc=P, out=P, sl=None, p=0.0, plan=None, rnp=1, ws=None, ws_bytes=0):
+    return lib.ffa_attention_diag(precision, B, H, Dh, Lmax, scale, t, q, k, v, kc, vc, out, sl, p,
+                                  C.byref(plan) if plan is not None else None, rnp, ws, ws_bytes,
+                                  None, None, None)
+
+
+def test_attention_argument_validation(lib):
+    wg = capi.make_plan(capi.FFA_LAUNCH_WORKGROUP, 4, 1, 1)
+    assert _attn(lib, precision=8, plan=wg) == 2          # dtype
+    assert _attn(lib, Dh=80, plan=wg) == 3                # head dim (80 is a reference size we do not ship)
+    assert _attn(lib, B=0, plan=wg) == 4
+    assert _attn(lib, H=-1, plan=wg) == 4
+    assert _attn(lib, t=-1, plan=wg) == 5
+    assert _attn(lib, t=128, Lmax=128, plan=wg) == 5      # the reference writes out of bounds here
+    assert _attn(lib, p=-0.5, plan=wg) == 10
+    assert _attn(lib, p=float("nan"), plan=wg) == 10
+    assert _attn(lib, q=None, plan=wg) == 1
+    assert _attn(lib, out=None, plan=wg) == 1
+    assert _attn(lib, kc=C.c_void_p(0x1008), plan=wg) == 6
+    # malformed plans
+    assert _attn(lib, plan=capi.make_plan(capi.FFA_LAUNCH_WORKGROUP, 3, 1, 1)) == 8
+    assert _attn(lib, plan=capi.make_plan(capi.FFA_LAUNCH_WORKGROUP, 4, 2, 1)) == 8
+    assert _attn(lib, plan=capi.make_plan(7, 4, 1, 1)) == 8
+    assert _attn(lib, t=100, plan=capi.make_plan(capi.FFA_LAUNCH_SPLIT, 4, 1, 1)) == 8   # 1 tile < 2 needed
+    assert _attn(lib, p=0.1, plan=capi.make_plan(capi.FFA_LAUNCH_SPLIT, 4, 2, 1)) == 8   # split is exact only
+    assert _attn(lib, plan=capi.make_plan(capi.FFA_LAUNCH_SPLIT, 16, 2, 1)) == 8
+    # split plan without / with too small a workspace
+    sp = capi.make_plan(capi.FFA_LAUNCH_SPLIT, 4, 2, 1)
+    assert _attn(lib, t=100, plan=sp) == 7
+    assert _attn(lib, t=100, plan=sp, ws=P, ws_bytes=64) == 7
+    # one-workgroup launch whose scores cannot fit in LDS
+    assert _attn(lib, t=60000, Lmax=65536, plan=wg) == 9
+
+
+def test_init_cache_argument_validation(lib):
+    f = lib.ffa_init_cache_f16
+    assert f(P, P, P, P, 1, 8, 4, 64, 2, None) == 4       # L > Lmax
+    assert f(P, P, P, P, 1, 8, 16, 96, 2, None) == 3
+    assert f(None, P, P, P, 1, 8, 16, 64, 2, None) == 1
+    assert f(P, P, None, P, 1, 8, 16, 64, 2, None) == 1
+    assert f(P, P, C.c_void_p(0x1004), P, 1, 8, 16, 64, 2, None) == 6
+    assert f(P, P, None, None, 1, 0, 16, 64, 2, None) == 0  # empty prompt: nothing to do
+    assert lib.ffa_workspace_init(None, 16, None) == 1
+
+
+def test_workspace_bytes_covers_every_plan(lib):
+    for (B, H, Dh, Lmax) in [(10, 32, 64, 1256), (1, 32, 64, 16384), (8, 16, 256, 2256), (16, 32, 64, 8256),
+                             (1, 1, 64, 1), (3, 5, 128, 700)]:
+        total = lib.ffa_workspace_bytes(B, H, Dh, Lmax)
+        assert total > 0
+        for prec in (16, 32):
+            for t in sorted({0, 1, 63, 64, Lmax // 2, Lmax - 1}):
+                for cus in (64, 256, 304):
+                    plan = capi.plan_launch(prec, B, H, Dh, t, 0.0, False, cus)
+                    bh = B * H
+                    need = -(-bh * 4 // 256) * 256
+                    if plan.n_splits > 1:
+                        need += -(-bh * plan.n_splits * 8 // 256) * 256 + bh * plan.n_splits * Dh * 4
+                    assert need <= total, (B, H, Dh, Lmax, t, plan)
+    assert lib.ffa_workspace_bytes(0, 1, 64, 8) == 0
+
+
+@pytest.mark.parametrize("prec", [16, 32])
+@pytest.mark.parametrize("Dh", [64, 128, 256])
+def test_planner_consistency(prec, Dh):
+    for B, H in [(1, 1), (1, 32), (2, 32), (10, 32), (16, 32), (64, 64)]:
+        for t in [0, 1, 31, 63, 64, 127, 999, 1000, 1255, 2047, 2048, 8191, 16383, 30000]:
+            ntiles = t // 64 + 1
+            for use_default in (False, True):
+                for p in (0.0, 1e-3):
+                    plan = capi.plan_launch(prec, B, H, Dh, t, p, use_default, 256)
+                    assert plan.threads_per_key == 1 and plan.keys_per_wave == 64
+                    assert plan.waves_per_wg in (1, 2, 4, 8, 16)
+                    assert plan.n_splits * plan.tiles_per_split >= ntiles      # every key covered
+                    if use_default or p > 0:
+                        assert plan.kind == capi.FFA_LAUNCH_WORKGROUP and plan.n_splits == 1
+                    else:
+                        assert plan.kind == capi.FFA_LAUNCH_SPLIT
+                        assert (plan.n_splits - 1) * plan.tiles_per_split < ntiles  # no empty split
+                        assert B * H * plan.n_splits <= 16384
+                        assert plan.waves_per_wg <= 8
+
+
+def test_planner_default_follows_length_table():
+    # kernel_launch_utils.h:147-154: 64 / 128 / 256 threads by prompt length
+    assert capi.plan_launch(16, 10, 32, 64, 10, 0.0, True).waves_per_wg == 1
+    assert capi.plan_launch(16, 10, 32, 64, 1000, 0.0, True).waves_per_wg == 2
+    assert capi.plan_launch(16, 10, 32, 64, 4096, 0.0, True).waves_per_wg == 4
+
+
+def test_planner_rejects_bad_input(lib):
+    plan = capi.LaunchPlan()
+    f = lib.ffa_plan_launch
+    assert f(8, 1, 1, 64, 10, 0.0, 0, 256, C.byref(plan)) == 2
+    assert f(16, 1, 1, 80, 10, 0.0, 0, 256, C.byref(plan)) == 3
+    assert f(16, 0, 1, 64, 10, 0.0, 0, 256, C.byref(plan)) == 4
+    assert f(16, 1, 1, 64, -1, 0.0, 0, 256, C.byref(plan)) == 5
+    assert f(16, 1, 1, 64, 10, -1.0, 0, 256, C.byref(plan)) == 10
+    assert f(16, 1, 1, 64, 10, 0.0, 0, 256, None) == 1
+    assert f(16, 1, 1, 64, 50000, 0.5, 0, 256, C.byref(plan)) == 9   # pruned: scores must fit LDS
+    assert f(16, 1, 1, 64, 50000, 0.0, 1, 256, C.byref(plan)) == 9
+
+
+def test_extension_imports_and_refuses_cpu_tensors():
+    import torch
+    from fastforwardattention_amd import FastForwardAttn
+    with pytest.raises(RuntimeError, match="GPU tensors"):
+        FastForwardAttn(torch.zeros(1, 1, 4, 64), torch.zeros(1, 1, 4, 64), 8, False)
+    import ff_attention  # the reference's module name resolves to the same extension
+    assert ff_attention.FastForwardAttn is FastForwardAttn
