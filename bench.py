@@ -1,0 +1,315 @@
+#!/usr/bin/env python3
+"""Benchmark of the decode-attention hot path on ONE MI355X.
+
+Headline workload (BASELINE.json configs[1], B = 10): OPT-1.3b-shaped iterative decode,
+32 heads x 64, fp16, KV cache prefilled with a 1000-token prompt (N(0,1) * 0.5), then
+t = 1000 -> 1255, fresh N(0,1) q/k/v, scale 1/8, p = 0.
+
+A "step" is ONE decode-attention call: one layer's cache, one new token for the whole
+batch.  OPT-1.3b has 24 layers, so the bench keeps 24 independent caches (2.5 GB) and
+step i works on cache i % 24 at t = 1000 + (i // 24) % 256: consecutive steps never touch
+the same cache, as in a real decoder, and the 103 MB of one cache cannot be served out of
+the 256 MB last-level cache.  The default K = 6144 steps is the full 256-token decode.
+
+Three timed legs over the same K steps, each bracketed by torch.cuda.synchronize() and
+HIP events recorded on the launch stream:
+  graph   the K launches captured once into a HIP graph and replayed (device-side rate,
+          no host gaps) -> `value`, `ms_per_step`, `roofline`
+  capi    K eager calls of ffa_attention_f16 through ctypes          -> `eager_capi_*`
+  ext     K eager calls of FastForwardAttn.attention (Python API)    -> `eager_ext_*`
+plus `cpu_baseline`: the fp32 torch restatement of the reference's torch_attn_func on the
+host cores, on a bounded sample of the same workload.
+
+Prints ONE JSON line.
+"""
+from __future__ import annotations
+
+import argparse
+import ctypes as C
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
+
+WORKLOADS = {
+    # name: B, H, Dh, prompt, gen, scale, layers (independent caches), dtype
+    "opt1.3b_b10": dict(B=10, H=32, Dh=64, prompt=1000, gen=256, scale=0.125, layers=24),
+    "opt1.3b_b5": dict(B=5, H=32, Dh=64, prompt=1000, gen=256, scale=0.125, layers=24),
+    "opt1.3b_b2": dict(B=2, H=32, Dh=64, prompt=1000, gen=256, scale=0.125, layers=24),
+    "opt1.3b_b1": dict(B=1, H=32, Dh=64, prompt=1000, gen=256, scale=0.125, layers=24),
+    "gptj_b8": dict(B=8, H=16, Dh=256, prompt=2000, gen=256, scale=0.0625, layers=8),
+    "long_b1_16k": dict(B=1, H=32, Dh=64, prompt=16384 - 128, gen=128, scale=0.125, layers=24),
+    "long_b1_8k": dict(B=1, H=32, Dh=64, prompt=8192 - 128, gen=128, scale=0.125, layers=24),
+    "long_b1_4k": dict(B=1, H=32, Dh=64, prompt=4096 - 128, gen=128, scale=0.125, layers=24),
+    "long_b1_2k": dict(B=1, H=32, Dh=64, prompt=2048 - 128, gen=128, scale=0.125, layers=24),
+    "long_b1_1k": dict(B=1, H=32, Dh=64, prompt=1024 - 128, gen=128, scale=0.125, layers=24),
+}
+
+
+def algorithmic_bytes(B, H, Dh, t, elem=2):
+    """K and V cache reads of the t cached keys: 2*B*H*Dh*sizeof(T)*t."""
+    return 2 * B * H * Dh * elem * t
+
+
+class Workload:
+    def __init__(self, name, use_default=False, plan_override=None):
+        import torch
+        from fastforwardattention_amd import capi
+        self.torch, self.capi = torch, capi
+        self.lib = capi.load()
+        self.name = name
+        w = WORKLOADS[name]
+        self.B, self.H, self.Dh = w["B"], w["H"], w["Dh"]
+        self.prompt, self.gen, self.scale, self.layers = w["prompt"], w["gen"], w["scale"], w["layers"]
+        self.Lmax = self.prompt + self.gen
+        self.use_default = use_default
+        self.plan_override = plan_override
+        dev = "cuda:0"
+        B, H, Dh, L, Lmax = self.B, self.H, self.Dh, self.prompt, self.Lmax
+        g = torch.Generator(device=dev).manual_seed(0)
+        self.kc, self.vc = [], []
+        for _ in range(self.layers):
+            K = (torch.randn(B, H, L, Dh, device=dev, generator=g) * 0.5).half()
+            V = (torch.randn(B, H, L, Dh, device=dev, generator=g) * 0.5).half()
+            kc = torch.empty(B, H, Dh // 8, Lmax, 8, dtype=torch.float16, device=dev)
+            vc = torch.empty(B, H, Lmax, Dh, dtype=torch.float16, device=dev)
+            capi.check(self.lib.ffa_init_cache_f16(kc.data_ptr(), vc.data_ptr(), K.data_ptr(), V.data_ptr(),
+                                                   B, L, Lmax, Dh, H, None), "ffa_init_cache_f16")
+            torch.cuda.synchronize()
+            self.kc.append(kc)
+            self.vc.append(vc)
+            del K, V
+        # a ring of fresh q/k/v tokens (N(0,1)), resident in HBM before the timed region
+        self.ring = 64
+        self.q = torch.randn(self.ring, B, H, Dh, device=dev, generator=g).half()
+        self.k = torch.randn(self.ring, B, H, Dh, device=dev, generator=g).half()
+        self.v = torch.randn(self.ring, B, H, Dh, device=dev, generator=g).half()
+        self.out = torch.empty(self.ring, B, H, Dh, dtype=torch.float16, device=dev)
+        nbytes = self.lib.ffa_workspace_bytes(B, H, Dh, Lmax)
+        self.ws = torch.zeros(nbytes, dtype=torch.uint8, device=dev)
+        self.ws_bytes = nbytes
+        self._plans = {}
+        torch.cuda.synchronize()
+
+    def t_of(self, i):
+        return self.prompt + (i // self.layers) % self.gen
+
+    def plan_for(self, t):
+        p = self._plans.get(t)
+        if p is None:
+            if self.plan_override is not None:
+                kind, waves, tps = self.plan_override[:3]
+                combine = self.plan_override[3] if len(self.plan_override) > 3 else 0
+                ntiles = t // 64 + 1
+                ns = 1 if kind == self.capi.FFA_LAUNCH_WORKGROUP else -(-ntiles // tps)
+                p = self.capi.make_plan(kind, waves, ns, ntiles if ns == 1 and kind == 0 else tps, combine)
+            else:
+                p = self.capi.plan_launch(16, self.B, self.H, self.Dh, t, 0.0, self.use_default,
+                                          self.lib.ffa_device_compute_units())
+            self._plans[t] = p
+        return p
+
+    def launch(self, i, stream_ptr):
+        """One step through the C ABI (no allocation, no sync)."""
+        t = self.t_of(i)
+        r, l = i % self.ring, i % self.layers
+        rc = self.lib.ffa_attention_f16(
+            self.B, self.H, self.Dh, self.Lmax, self.scale, t,
+            self.q[r].data_ptr(), self.k[r].data_ptr(), self.v[r].data_ptr(),
+            self.kc[l].data_ptr(), self.vc[l].data_ptr(), self.out[r].data_ptr(), None, 0.0,
+            C.byref(self.plan_for(t)), 1, self.ws.data_ptr(), self.ws_bytes, stream_ptr)
+        if rc != 0:
+            raise RuntimeError(f"ffa_attention_f16 failed: {self.capi.status_string(rc)}")
+
+    def mean_bytes(self, steps):
+        return sum(algorithmic_bytes(self.B, self.H, self.Dh, self.t_of(i)) for i in range(steps)) / steps
+
+
+def time_region(torch, fn):
+    """fn() enqueues work on the current stream; returns elapsed ms between HIP events."""
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    fn()
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1)
+
+
+def run_graph(wl, steps, warmup):
+    torch = wl.torch
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):          # warm-up on the capture stream, eager
+        for i in range(warmup):
+            wl.launch(i, side.cuda_stream)
+    side.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        sp = torch.cuda.current_stream().cuda_stream
+        for i in range(steps):
+            wl.launch(i, sp)
+    graph.replay()                          # one untimed replay
+    torch.cuda.synchronize()
+    best = None
+    for _ in range(3):
+        ms = time_region(torch, graph.replay)
+        best = ms if best is None else min(best, ms)
+    return best
+
+
+def run_capi(wl, steps, warmup):
+    torch = wl.torch
+    sp = torch.cuda.current_stream().cuda_stream
+    for i in range(warmup):
+        wl.launch(i, sp)
+
+    def body():
+        for i in range(steps):
+            wl.launch(i, sp)
+    return time_region(torch, body)
+
+
+def run_ext(wl, steps, warmup):
+    """The Python API on one object per layer, built over the same caches."""
+    torch = wl.torch
+    from fastforwardattention_amd import FastForwardAttn
+    B, H, Dh = wl.B, wl.H, wl.Dh
+    dummy = torch.zeros(B, H, 1, Dh, dtype=torch.float16, device="cuda:0")
+    obj = FastForwardAttn(dummy, dummy, wl.Lmax, wl.use_default)  # its own caches are unused
+    def step(i):
+        r, l = i % wl.ring, i % wl.layers
+        return obj.attention(wl.q[r], wl.k[r], wl.v[r], wl.kc[l], wl.vc[l], wl.scale, wl.t_of(i), 0.0)
+    for i in range(warmup):
+        step(i)
+
+    def body():
+        for i in range(steps):
+            step(i)
+    return time_region(torch, body)
+
+
+def cpu_baseline(wl, budget_s=15.0, max_steps=64):
+    """The reference's CPU path restated (oracle/torch_attn.py) on the host cores, on the
+    first steps of the same workload (one layer's cache), bounded by a time budget."""
+    import torch
+    from oracle.torch_attn import CpuDecodeBaseline
+    B, H, Dh, L = wl.B, wl.H, wl.Dh, wl.prompt
+    g = torch.Generator().manual_seed(0)
+    K = torch.randn(B, H, L, Dh, generator=g) * 0.5
+    V = torch.randn(B, H, L, Dh, generator=g) * 0.5
+    base = CpuDecodeBaseline(K, V, wl.Lmax)
+    toks = [tuple(torch.randn(B, H, Dh, generator=g) for _ in range(3)) for _ in range(8)]
+    for i in range(3):
+        q, k, v = toks[i % 8]
+        base.attention(q, k, v, wl.scale, L + i)
+    times, t0 = [], time.perf_counter()
+    i = 0
+    while i < max_steps and (time.perf_counter() - t0) < budget_s:
+        q, k, v = toks[i % 8]
+        s = time.perf_counter()
+        base.attention(q, k, v, wl.scale, L + 3 + i)
+        times.append(time.perf_counter() - s)
+        i += 1
+    mean_s = sum(times) / len(times)
+    t_mid = L + 3 + len(times) // 2
+    gbs = algorithmic_bytes(B, H, Dh, t_mid, elem=4) / mean_s / 1e9
+    return {
+        "value": round(gbs, 3), "unit": "GB/s", "cores": torch.get_num_threads(),
+        "host_cpus": os.cpu_count(), "kind": "port",
+        "us_per_step": round(mean_s * 1e6, 1),
+        "sample": (f"{len(times)} decode steps of {wl.name} (one layer, t={L + 3}..{L + 2 + len(times)}), "
+                   "fp32 torch bmm/softmax/bmm over a pre-allocated cache; bytes counted at 4 B/element"),
+    }
+
+
+def load_traffic(name):
+    """HBM bytes per launch measured with rocprofv3 --pmc (FETCH_SIZE, WRITE_SIZE), kept in
+    profiles/traffic.json by hand after a counter run; None when not measured."""
+    path = os.path.join(ROOT, "profiles", "traffic.json")
+    try:
+        with open(path) as f:
+            return json.load(f).get(name)
+    except (OSError, ValueError):
+        return None
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=6144)
+    ap.add_argument("--warmup", type=int, default=240)
+    ap.add_argument("--workload", default="opt1.3b_b10", choices=sorted(WORKLOADS))
+    ap.add_argument("--default-launch", action="store_true", help="use_default_kernel_launch=True")
+    ap.add_argument("--plan", default=None, help="kind,waves,tiles_per_split[,combine] (kind: 0 workgroup, 1 split; combine: 0 fused, 1 kernel)")
+    ap.add_argument("--legs", default="graph,capi,ext", help="comma list of graph,capi,ext")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on exactly one GPU (one process, one MI355X); "
+              f"--gpus {args.gpus} is not supported.", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible; the hot path has no CPU fallback.", file=sys.stderr)
+        sys.exit(3)
+
+    plan_override = tuple(int(x) for x in args.plan.split(",")) if args.plan else None
+    wl = Workload(args.workload, use_default=args.default_launch, plan_override=plan_override)
+    steps, warmup = args.steps, args.warmup
+    legs = [x for x in args.legs.split(",") if x]
+    mean_b = wl.mean_bytes(steps)
+
+    res = {}
+    if "graph" in legs:
+        res["graph"] = run_graph(wl, steps, warmup)
+    if "capi" in legs:
+        res["capi"] = run_capi(wl, steps, warmup)
+    if "ext" in legs:
+        res["ext"] = run_ext(wl, steps, warmup)
+    primary = "graph" if "graph" in res else legs[0]
+    ms = res[primary]
+    us_step = ms * 1e3 / steps
+    gbs = mean_b / (us_step * 1e-6) / 1e9
+
+    plan0 = wl.plan_for(wl.t_of(0))
+    out = {
+        "metric": "KV-cache HBM GB/s (decode attention, OPT-1.3b shape B=10, t=1000->1256)"
+                  if args.workload == "opt1.3b_b10" else f"KV-cache HBM GB/s ({args.workload})",
+        "value": round(gbs, 1), "unit": "GB/s", "n_gpus": 1, "steps": steps, "warmup": warmup,
+        "ms_per_step": round(us_step / 1e3, 6), "us_per_step": round(us_step, 3),
+        "tokens_per_s": round(wl.B / (us_step * 1e-6), 1),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f16 (fp32 accumulate)", "data": "synthetic",
+        "config": {"workload": f"{args.workload}: B={wl.B} H={wl.H} Dh={wl.Dh} fp16 prompt={wl.prompt} "
+                               f"t={wl.prompt}->{wl.prompt + min(wl.gen, -(-steps // wl.layers))} p=0 "
+                               f"scale={wl.scale}; step = one attention call on one of {wl.layers} "
+                               "independent layer caches",
+                   "timing_leg": primary,
+                   "launch_plan_at_first_step": repr(plan0)},
+        "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(gbs / HBM_PEAK_GBS, 4),
+                     "traffic": load_traffic(args.workload),
+                     "algorithmic_bytes_per_launch": round(mean_b),
+                     "kernel": "ffa_decode_split_kernel" if plan0.kind == 1 else "ffa_decode_wg_kernel",
+                     "launch_us": round(us_step, 3)},
+    }
+    for leg in ("capi", "ext"):
+        if leg in res and leg != primary:
+            u = res[leg] * 1e3 / steps
+            out[f"eager_{leg}_us_per_step"] = round(u, 3)
+            out[f"eager_{leg}_GBps"] = round(mean_b / (u * 1e-6) / 1e9, 1)
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline(wl)
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -25,10 +25,19 @@ __all__ = ["FastForwardAttn", "ff_attention", "capi"]
 
 
 def _load_extension():
+    """Load the compiled module once, under the reference's top-level name `ff_attention`
+    (so that `from ff_attention import FastForwardAttn` and this package share one module
+    object and one pybind11 type registration)."""
+    if "ff_attention" in sys.modules:
+        return sys.modules["ff_attention"]
     try:
         import torch  # noqa: F401  (libtorch must be loaded before the extension)
-        return importlib.import_module("fastforwardattention_amd.ff_attention")
-    except ImportError as exc:  # pragma: no cover - exercised only on broken installs
+        sys.path.insert(0, _PKG_DIR)
+        try:
+            return importlib.import_module("ff_attention")
+        finally:
+            sys.path.remove(_PKG_DIR)
+    except ImportError as exc:
         raise ImportError(
             "fastforwardattention_amd: the compiled extension ff_attention (and libffa_hip.so) "
             "is not built or cannot be loaded; run `python -m fastforwardattention_amd._build`. "
@@ -38,9 +47,7 @@ def _load_extension():
 def __getattr__(name):
     # Lazy so that `import fastforwardattention_amd._build` works before anything is built.
     if name == "ff_attention":
-        mod = _load_extension()
-        sys.modules.setdefault("ff_attention", mod)  # reference spelling: from ff_attention import ...
-        return mod
+        return _load_extension()
     if name == "FastForwardAttn":
         return __getattr__("ff_attention").FastForwardAttn
     if name == "capi":

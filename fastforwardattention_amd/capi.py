@@ -16,6 +16,8 @@ FFA_PRECISION_F16 = 16
 FFA_PRECISION_F32 = 32
 FFA_LAUNCH_WORKGROUP = 0
 FFA_LAUNCH_SPLIT = 1
+FFA_COMBINE_FUSED = 0
+FFA_COMBINE_KERNEL = 1
 
 STATUS_NAMES = {
     0: "FFA_OK", 1: "FFA_ERR_NULL_POINTER", 2: "FFA_ERR_DTYPE", 3: "FFA_ERR_HEAD_DIM",
@@ -29,7 +31,7 @@ class LaunchPlan(C.Structure):
     """struct ffa_launch_plan."""
     _fields_ = [("kind", C.c_int32), ("waves_per_wg", C.c_int32), ("threads_per_key", C.c_int32),
                 ("keys_per_wave", C.c_int32), ("n_splits", C.c_int32),
-                ("tiles_per_split", C.c_int32), ("reserved", C.c_int32 * 2)]
+                ("tiles_per_split", C.c_int32), ("combine", C.c_int32), ("reserved", C.c_int32)]
 
     def as_tuple(self):
         return (self.kind, self.waves_per_wg, self.threads_per_key, self.keys_per_wave,
@@ -39,7 +41,7 @@ class LaunchPlan(C.Structure):
         kind = {0: "workgroup", 1: "split"}.get(self.kind, str(self.kind))
         return (f"LaunchPlan(kind={kind}, waves_per_wg={self.waves_per_wg}, "
                 f"threads_per_key={self.threads_per_key}, n_splits={self.n_splits}, "
-                f"tiles_per_split={self.tiles_per_split})")
+                f"tiles_per_split={self.tiles_per_split}, combine={self.combine})")
 
 
 _vp, _i, _f, _sz = C.c_void_p, C.c_int, C.c_float, C.c_size_t
@@ -97,8 +99,8 @@ def plan_launch(precision, B, H, Dh, t, p=0.0, use_default=False, compute_units=
     return plan
 
 
-def make_plan(kind, waves_per_wg, n_splits, tiles_per_split) -> LaunchPlan:
+def make_plan(kind, waves_per_wg, n_splits, tiles_per_split, combine=0) -> LaunchPlan:
     plan = LaunchPlan()
     plan.kind, plan.waves_per_wg, plan.threads_per_key, plan.keys_per_wave = kind, waves_per_wg, 1, 64
-    plan.n_splits, plan.tiles_per_split = n_splits, tiles_per_split
+    plan.n_splits, plan.tiles_per_split, plan.combine = n_splits, tiles_per_split, combine
     return plan

@@ -22,13 +22,18 @@ __device__ __forceinline__ float dpp_f32(float x) {
         float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), CTRL, 0xf, 0xf, false));
 }
 
+// __builtin_amdgcn_readlane is typed int -> int: move the bits, not the value.
+__device__ __forceinline__ float readlane_f32(float x, int lane) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, x), lane));
+}
+
 __device__ __forceinline__ float wave_max(float x) {
     x = fmaxf(x, dpp_f32<0xB1>(x));
     x = fmaxf(x, dpp_f32<0x4E>(x));
     x = fmaxf(x, dpp_f32<0x141>(x));
     x = fmaxf(x, dpp_f32<0x140>(x));
-    const float a = __builtin_amdgcn_readlane(x, 0), b = __builtin_amdgcn_readlane(x, 16);
-    const float c = __builtin_amdgcn_readlane(x, 32), d = __builtin_amdgcn_readlane(x, 48);
+    const float a = readlane_f32(x, 0), b = readlane_f32(x, 16);
+    const float c = readlane_f32(x, 32), d = readlane_f32(x, 48);
     return fmaxf(fmaxf(a, b), fmaxf(c, d));
 }
 
@@ -37,8 +42,8 @@ __device__ __forceinline__ float wave_sum(float x) {
     x += dpp_f32<0x4E>(x);
     x += dpp_f32<0x141>(x);
     x += dpp_f32<0x140>(x);
-    const float a = __builtin_amdgcn_readlane(x, 0), b = __builtin_amdgcn_readlane(x, 16);
-    const float c = __builtin_amdgcn_readlane(x, 32), d = __builtin_amdgcn_readlane(x, 48);
+    const float a = readlane_f32(x, 0), b = readlane_f32(x, 16);
+    const float c = readlane_f32(x, 32), d = readlane_f32(x, 48);
     return (a + b) + (c + d);
 }
 

@@ -49,6 +49,7 @@ struct DecodeParams {
     int right_or_no_padding;
     int n_splits, tiles_per_split;
     int bh_total;
+    int combine;  // FFA_COMBINE_*
 };
 
 // Per-(b) bounds, attention.cu:805-817.  tlen = slot of the new token = number of cached
@@ -118,6 +119,14 @@ struct Geo {
 // row group rg = lane/LPR, the NCH consecutive floats [rg*NCH, rg*NCH+NCH) = keys j*RPI+rg.
 template <int NCH, int RPI>
 __device__ __forceinline__ int stage_slot(int k) { return (k % RPI) * NCH + k / RPI; }
+
+// Words exchanged between workgroups of one launch: device-scope relaxed atomics.
+__device__ __forceinline__ void publish(float* p, float v) {
+    __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ float acquire(const float* p) {
+    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
 
 // ---------------------------------------------------------------------------------------
 // Sequence-split exact decode (p == 0).
@@ -196,12 +205,12 @@ __global__ void __launch_bounds__(NW * 64) ffa_decode_split_kernel(const DecodeP
         load_v_group(vv, tile, 0);
 
         const bool valid = key <= tlen && key >= first;
-        s = valid ? s * P.scale_log2e : -INFINITY;
-
-        const float m_new = fmaxf(m_run, wave_max(s));
+        const float m_new = fmaxf(m_run, wave_max(valid ? s * P.scale_log2e : -INFINITY));
         // m_new == -inf only while every key seen so far is masked: acc, l are still 0.
         const float alpha = (m_new == -INFINITY) ? 1.f : __builtin_amdgcn_exp2f(m_run - m_new);
-        const float pr = valid ? __builtin_amdgcn_exp2f(s - m_new) : 0.f;
+        // One rounding for s*c - m: the rounding of m itself is a common factor of every
+        // weight and cancels in the normalisation.
+        const float pr = valid ? __builtin_amdgcn_exp2f(fmaf(s, P.scale_log2e, -m_new)) : 0.f;
         l_run = l_run * alpha + pr;
         m_run = m_new;
 
@@ -257,40 +266,77 @@ __global__ void __launch_bounds__(NW * 64) ffa_decode_split_kernel(const DecodeP
             o += wgt[w] * ow;
         }
         if (P.n_splits == 1) store_out(out, d, L > 0.f ? o / L : 0.f);
+        else if (P.combine == FFA_COMBINE_FUSED) publish(&wa[d], o);
         else wa[d] = o;
     }
     if (P.n_splits == 1) return;
+    if (P.combine != FFA_COMBINE_FUSED) {
+        // A second kernel merges: plain stores would do, the kernel boundary publishes them.
+        if (tid == 0) {
+            float* ml = P.ws_ml + ((size_t)bh * P.n_splits + split) * 2;
+            ml[0] = M;
+            ml[1] = L;
+        }
+        return;
+    }
 
     // ---- publish the partial; the last workgroup to arrive merges all splits ----
+    // No device-scope fence here: on this part such a fence writes back / invalidates a
+    // whole L2 and costs far more than the kernel itself.  Instead every word that crosses
+    // workgroups is moved with device-scope atomic accesses, which the hardware performs
+    // at the level all XCDs share, so nothing needs flushing.  Order: each thread's
+    // published stores are complete before the workgroup barrier (the barrier waits for
+    // outstanding memory operations), the arrival counter is bumped after it, and the
+    // merging workgroup reads the partials only after it has seen the final count.
     if (tid == 0) {
         float* ml = P.ws_ml + ((size_t)bh * P.n_splits + split) * 2;
-        ml[0] = M;
-        ml[1] = L;
+        publish(&ml[0], M);
+        publish(&ml[1], L);
     }
-    __threadfence();
     __syncthreads();
     if (tid == 0) {
-        const unsigned prev = atomicAdd(&P.ws_cnt[bh], 1u);
+        const unsigned prev =
+            __hip_atomic_fetch_add(&P.ws_cnt[bh], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         s_last = (prev == (unsigned)(P.n_splits - 1));
     }
     __syncthreads();
     if (!s_last) return;
-    __threadfence();
 
     const float* ml = P.ws_ml + (size_t)bh * P.n_splits * 2;
     float Mg = -INFINITY;
-    for (int s = 0; s < P.n_splits; ++s) Mg = fmaxf(Mg, __builtin_nontemporal_load(&ml[2 * s]));
+    for (int s = 0; s < P.n_splits; ++s) Mg = fmaxf(Mg, acquire(&ml[2 * s]));
     for (int d = tid; d < DH; d += NW * 64) {
         float o = 0.f, Lg = 0.f;
         for (int s = 0; s < P.n_splits; ++s) {
-            const float ms = __builtin_nontemporal_load(&ml[2 * s]);
+            const float ms = acquire(&ml[2 * s]);
             const float w = (ms == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(ms - Mg);
-            Lg += w * __builtin_nontemporal_load(&ml[2 * s + 1]);
-            o += w * __builtin_nontemporal_load(&P.ws_acc[((size_t)bh * P.n_splits + s) * DH + d]);
+            Lg += w * acquire(&ml[2 * s + 1]);
+            o += w * acquire(&P.ws_acc[((size_t)bh * P.n_splits + s) * DH + d]);
         }
         store_out(out, d, Lg > 0.f ? o / Lg : 0.f);
     }
-    if (tid == 0) P.ws_cnt[bh] = 0u;  // ready for the next launch on this stream
+    // Ready for the next launch on this stream (kernel boundaries order this store).
+    if (tid == 0) __hip_atomic_store(&P.ws_cnt[bh], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// Merge kernel of FFA_COMBINE_KERNEL: one wave per (b,h), log-sum-exp over the splits.
+template <typename T, int DH>
+__global__ void __launch_bounds__(64) ffa_merge_splits_kernel(const DecodeParams P) {
+    const int bh = blockIdx.x, tid = threadIdx.x;
+    const float* ml = P.ws_ml + (size_t)bh * P.n_splits * 2;
+    float Mg = -INFINITY;
+    for (int s = 0; s < P.n_splits; ++s) Mg = fmaxf(Mg, ml[2 * s]);
+    T* out = reinterpret_cast<T*>(P.out) + (size_t)bh * DH;
+    for (int d = tid; d < DH; d += 64) {
+        float o = 0.f, Lg = 0.f;
+        for (int s = 0; s < P.n_splits; ++s) {
+            const float ms = ml[2 * s];
+            const float w = (ms == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(ms - Mg);
+            Lg += w * ml[2 * s + 1];
+            o += w * P.ws_acc[((size_t)bh * P.n_splits + s) * DH + d];
+        }
+        store_out(out, d, Lg > 0.f ? o / Lg : 0.f);
+    }
 }
 
 // ---------------------------------------------------------------------------------------
@@ -339,15 +385,14 @@ __global__ void __launch_bounds__(NW * 64) ffa_decode_wg_kernel(const DecodePara
 
     if (wave == 0) append_new_token<NCH>(kc_bh, vc_bh, knew, vnew, tlen, P.Lmax, lane);
 
-    // ---- phase 1: scores (exp2 domain) to LDS, running max ----
+    // ---- phase 1: raw scores to LDS, running max (exp2 domain) ----
     float mx = -INFINITY;
     for (int tile = tile_lo + wave; tile < ntiles; tile += NW) {
         const int key = tile * kWave + lane;
         float s = tile_qk<T, NCH, G::Q_LDS>(kc_bh, knew, key, tlen, P.Lmax, q_reg, s_q);
         const bool valid = key <= tlen && key >= first;
-        s = valid ? s * P.scale_log2e : -INFINITY;
-        s_sc[key] = s;
-        mx = fmaxf(mx, s);
+        s_sc[key] = valid ? s : -INFINITY;  // raw dot product; scaled inside the exp2 below
+        mx = fmaxf(mx, valid ? s * P.scale_log2e : -INFINITY);
     }
     mx = wave_max(mx);
     if (lane == 0) s_red[wave] = mx;
@@ -362,7 +407,9 @@ __global__ void __launch_bounds__(NW * 64) ffa_decode_wg_kernel(const DecodePara
     // ---- phase 2: e_i = exp(s_i - max), sum ----
     float sum = 0.f;
     for (int i = tile_lo * kWave + tid; i < ntiles * kWave; i += NT) {
-        const float e = __builtin_amdgcn_exp2f(s_sc[i] - M);  // exp2(-inf) = 0 for masked keys
+        const float sr = s_sc[i];
+        // one rounding for s*c - M; masked keys (-inf) give exactly 0
+        const float e = (sr == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(fmaf(sr, P.scale_log2e, -M));
         s_sc[i] = e;
         sum += e;
     }
@@ -510,6 +557,8 @@ static int launch_split(const DecodeParams& P, hipStream_t st) {
     const int groups = (P.bh_total + 7) / 8;
     const dim3 grid((unsigned)(groups * 8 * P.n_splits));
     hipLaunchKernelGGL((ffa_decode_split_kernel<T, DH, NW>), grid, dim3(NW * 64), 0, st, P);
+    if (P.n_splits > 1 && P.combine == FFA_COMBINE_KERNEL)
+        hipLaunchKernelGGL((ffa_merge_splits_kernel<T, DH>), dim3((unsigned)P.bh_total), dim3(64), 0, st, P);
     return check_launch();
 }
 
@@ -579,6 +628,7 @@ int launch_decode(const DecodeArgs& a, const ffa_launch_plan& plan, const Worksp
     P.right_or_no_padding = a.right_or_no_padding;
     P.n_splits = plan.n_splits; P.tiles_per_split = plan.tiles_per_split;
     P.bh_total = a.B * a.H;
+    P.combine = plan.combine;
     hipStream_t st = reinterpret_cast<hipStream_t>(a.stream);
     if (a.precision == FFA_PRECISION_F16) return dispatch_head_dim<uint16_t>(P, a.Dh, plan, st);
     return dispatch_head_dim<float>(P, a.Dh, plan, st);

@@ -27,7 +27,8 @@ static void fill(ffa_launch_plan* plan, int kind, int waves, int n_splits, int t
     plan->keys_per_wave = kTileKeys;
     plan->n_splits = n_splits;
     plan->tiles_per_split = tiles_per_split;
-    plan->reserved[0] = plan->reserved[1] = 0;
+    plan->combine = FFA_COMBINE_FUSED;
+    plan->reserved = 0;
 }
 
 // Largest power-of-two wave count (<= 16) whose score buffer + merge buffer fit in LDS and
@@ -89,6 +90,7 @@ int validate_plan(const ffa_launch_plan& plan, int precision, int t, float p) {
     if (w != 1 && w != 2 && w != 4 && w != 8 && w != 16) return FFA_ERR_PLAN;
     if (plan.threads_per_key != 1 || plan.keys_per_wave != kTileKeys) return FFA_ERR_PLAN;
     if (plan.n_splits < 1 || plan.n_splits > kMaxSplits || plan.tiles_per_split < 1) return FFA_ERR_PLAN;
+    if (plan.combine != FFA_COMBINE_FUSED && plan.combine != FFA_COMBINE_KERNEL) return FFA_ERR_PLAN;
     const int ntiles = num_tiles(t);
     switch (plan.kind) {
         case FFA_LAUNCH_WORKGROUP:

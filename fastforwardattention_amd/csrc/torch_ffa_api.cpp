@@ -13,8 +13,10 @@
 //     length (torch_ffa_api.cpp:176).
 #include <torch/extension.h>
 
-#include <c10/hip/HIPGuard.h>
-#include <c10/hip/HIPStream.h>
+// PyTorch-ROCm presents HIP devices under the device type "cuda"; these are the guard and
+// stream accessors that understand that.
+#include <ATen/hip/impl/HIPGuardImplMasqueradingAsCUDA.h>
+#include <ATen/hip/impl/HIPStreamMasqueradingAsCUDA.h>
 
 #include <tuple>
 #include <utility>
@@ -36,7 +38,7 @@ int precision_of(const torch::Tensor& x) {
 }
 
 void* stream_of(const torch::Tensor& x) {
-    return static_cast<void*>(c10::hip::getCurrentHIPStream(x.device().index()).stream());
+    return static_cast<void*>(c10::hip::getCurrentHIPStreamMasqueradingAsCUDA(x.device().index()).stream());
 }
 
 struct CacheDims {
@@ -90,7 +92,7 @@ struct FastForwardAttn {
         const int x = 16 / (int)K.element_size();
         TORCH_CHECK(Dh % x == 0, "ff_attention: head dim must be a multiple of ", x);
 
-        c10::hip::HIPGuard guard(K.device());
+        c10::hip::HIPGuardMasqueradingAsCUDA guard(K.device());
         K = K.contiguous();
         V = V.contiguous();
         k_cache = torch::empty({B, H, Dh / x, max_timesteps, x}, K.options());
@@ -150,7 +152,7 @@ struct FastForwardAttn {
     }
 
     // Not in the reference: the plan the next call at (t, p) would use, as
-    // (kind, waves_per_wg, threads_per_key, keys_per_wave, n_splits, tiles_per_split).
+    // (kind, waves_per_wg, threads_per_key, keys_per_wave, n_splits, tiles_per_split, combine).
     std::vector<int> launch_plan(int curr_timestep, float prob_thresh) {
         const CacheDims d = dims_of(k_cache, v_cache);
         ffa_launch_plan plan;
@@ -158,7 +160,7 @@ struct FastForwardAttn {
                                      ft_kernel_launch ? 1 : 0, 0, &plan),
                      "launch planning");
         return {plan.kind, plan.waves_per_wg, plan.threads_per_key, plan.keys_per_wave, plan.n_splits,
-                plan.tiles_per_split};
+                plan.tiles_per_split, plan.combine};
     }
 
     torch::Tensor k_cache;
@@ -186,7 +188,7 @@ private:
         TORCH_CHECK(t >= 0 && t < d.Lmax, "ff_attention: timestep ", t, " outside the cache [0, ",
                     d.Lmax, ")");
         const int64_t numel = (int64_t)d.B * d.H * d.Dh;
-        c10::hip::HIPGuard guard(kc.device());
+        c10::hip::HIPGuardMasqueradingAsCUDA guard(kc.device());
         torch::Tensor q = token_input(q_in, kc, numel, "q");
         torch::Tensor k = token_input(k_in, kc, numel, "k");
         torch::Tensor v = token_input(v_in, kc, numel, "v");

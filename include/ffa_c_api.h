@@ -59,6 +59,10 @@ typedef enum ffa_status {
 #define FFA_LAUNCH_SPLIT 1      /* sequence split over n_splits workgroups per (batch,      */
                                 /* head), online softmax, last-arriver combine; p == 0 only */
 
+/* How the partial (max, sum, acc[Dh]) results of a split launch are merged. */
+#define FFA_COMBINE_FUSED 0     /* by the last workgroup of each (batch, head) to arrive     */
+#define FFA_COMBINE_KERNEL 1    /* by a second, small kernel on the same stream              */
+
 /* Replaces the (tpb, tpv, tpk) triple of kernel_launch_utils.h:135-180. */
 typedef struct ffa_launch_plan {
     int32_t kind;             /* FFA_LAUNCH_*                                              */
@@ -67,7 +71,8 @@ typedef struct ffa_launch_plan {
     int32_t keys_per_wave;    /* 64 / threads_per_key                                      */
     int32_t n_splits;         /* workgroups per (batch, head); 1 for FFA_LAUNCH_WORKGROUP  */
     int32_t tiles_per_split;  /* 64-key tiles each split walks                             */
-    int32_t reserved[2];
+    int32_t combine;          /* FFA_COMBINE_*: how split partials are merged              */
+    int32_t reserved;
 } ffa_launch_plan;
 
 int ffa_api_version(void);

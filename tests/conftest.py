@@ -6,6 +6,11 @@ import pytest
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
+# The reference's import line is `from ff_attention import FastForwardAttn`; the compiled
+# module of that name lives in the package directory.
+_EXT_DIR = os.path.join(ROOT, "fastforwardattention_amd")
+if _EXT_DIR not in sys.path:
+    sys.path.append(_EXT_DIR)
 
 
 def pytest_configure(config):

@@ -76,6 +76,7 @@ def test_attention_argument_validation(lib):
     assert _attn(lib, plan=capi.make_plan(capi.FFA_LAUNCH_WORKGROUP, 3, 1, 1)) == 8
     assert _attn(lib, plan=capi.make_plan(capi.FFA_LAUNCH_WORKGROUP, 4, 2, 1)) == 8
     assert _attn(lib, plan=capi.make_plan(7, 4, 1, 1)) == 8
+    assert _attn(lib, plan=capi.make_plan(capi.FFA_LAUNCH_SPLIT, 4, 1, 1, combine=5)) == 8
     assert _attn(lib, t=100, plan=capi.make_plan(capi.FFA_LAUNCH_SPLIT, 4, 1, 1)) == 8   # 1 tile < 2 needed
     assert _attn(lib, p=0.1, plan=capi.make_plan(capi.FFA_LAUNCH_SPLIT, 4, 2, 1)) == 8   # split is exact only
     assert _attn(lib, plan=capi.make_plan(capi.FFA_LAUNCH_SPLIT, 16, 2, 1)) == 8
