@@ -106,9 +106,11 @@ class Workload:
             if self.plan_override is not None:
                 kind, waves, tps = self.plan_override[:3]
                 combine = self.plan_override[3] if len(self.plan_override) > 3 else 0
+                whole = self.plan_override[4] if len(self.plan_override) > 4 else 0
                 ntiles = t // 64 + 1
                 ns = 1 if kind == self.capi.FFA_LAUNCH_WORKGROUP else -(-ntiles // tps)
-                p = self.capi.make_plan(kind, waves, ns, ntiles if ns == 1 and kind == 0 else tps, combine)
+                p = self.capi.make_plan(kind, waves, ns, ntiles if ns == 1 and kind == 0 else tps, combine,
+                                        whole)
             else:
                 p = self.capi.plan_launch(16, self.B, self.H, self.Dh, t, 0.0, self.use_default,
                                           self.lib.ffa_device_compute_units())
@@ -247,7 +249,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=240)
     ap.add_argument("--workload", default="opt1.3b_b10", choices=sorted(WORKLOADS))
     ap.add_argument("--default-launch", action="store_true", help="use_default_kernel_launch=True")
-    ap.add_argument("--plan", default=None, help="kind,waves,tiles_per_split[,combine] (kind: 0 workgroup, 1 split; combine: 0 fused, 1 kernel)")
+    ap.add_argument("--plan", default=None, help="kind,waves,tiles_per_split[,combine[,whole_heads]] (kind: 0 workgroup, 1 split; combine: 0 fused, 1 kernel)")
     ap.add_argument("--legs", default="graph,capi,ext", help="comma list of graph,capi,ext")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     args = ap.parse_args()

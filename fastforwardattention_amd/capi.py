@@ -31,17 +31,18 @@ class LaunchPlan(C.Structure):
     """struct ffa_launch_plan."""
     _fields_ = [("kind", C.c_int32), ("waves_per_wg", C.c_int32), ("threads_per_key", C.c_int32),
                 ("keys_per_wave", C.c_int32), ("n_splits", C.c_int32),
-                ("tiles_per_split", C.c_int32), ("combine", C.c_int32), ("reserved", C.c_int32)]
+                ("tiles_per_split", C.c_int32), ("combine", C.c_int32), ("whole_heads", C.c_int32)]
 
     def as_tuple(self):
         return (self.kind, self.waves_per_wg, self.threads_per_key, self.keys_per_wave,
-                self.n_splits, self.tiles_per_split)
+                self.n_splits, self.tiles_per_split, self.combine, self.whole_heads)
 
     def __repr__(self):
         kind = {0: "workgroup", 1: "split"}.get(self.kind, str(self.kind))
         return (f"LaunchPlan(kind={kind}, waves_per_wg={self.waves_per_wg}, "
                 f"threads_per_key={self.threads_per_key}, n_splits={self.n_splits}, "
-                f"tiles_per_split={self.tiles_per_split}, combine={self.combine})")
+                f"tiles_per_split={self.tiles_per_split}, combine={self.combine}, "
+                f"whole_heads={self.whole_heads})")
 
 
 _vp, _i, _f, _sz = C.c_void_p, C.c_int, C.c_float, C.c_size_t
@@ -99,8 +100,9 @@ def plan_launch(precision, B, H, Dh, t, p=0.0, use_default=False, compute_units=
     return plan
 
 
-def make_plan(kind, waves_per_wg, n_splits, tiles_per_split, combine=0) -> LaunchPlan:
+def make_plan(kind, waves_per_wg, n_splits, tiles_per_split, combine=0, whole_heads=0) -> LaunchPlan:
     plan = LaunchPlan()
     plan.kind, plan.waves_per_wg, plan.threads_per_key, plan.keys_per_wave = kind, waves_per_wg, 1, 64
     plan.n_splits, plan.tiles_per_split, plan.combine = n_splits, tiles_per_split, combine
+    plan.whole_heads = whole_heads
     return plan

@@ -43,21 +43,24 @@ int run_decode(const DecodeArgs& a, const ffa_launch_plan* user_plan, void* work
             st = plan_launch(a.precision, a.B, a.H, a.Dh, a.t, 1.f, 0, 256, &plan);
         if (st != FFA_OK) return st;
     }
-    st = validate_plan(plan, a.precision, a.t, a.p);
+    st = validate_plan(plan, a.precision, a.B * a.H, a.t, a.p);
     if (st != FFA_OK) return st;
     if (diag && plan.kind != FFA_LAUNCH_WORKGROUP) return FFA_ERR_PLAN;
 
     WorkspaceView ws = {nullptr, nullptr, nullptr};
-    if (plan.kind == FFA_LAUNCH_SPLIT && plan.n_splits > 1) {
-        const int bh = a.B * a.H;
-        if (workspace == nullptr || workspace_bytes < workspace_bytes_for(bh, a.Dh, plan.n_splits))
+    const int bh = a.B * a.H;
+    const int split_heads = bh - plan.whole_heads;
+    if (plan.kind == FFA_LAUNCH_SPLIT && plan.n_splits > 1 && split_heads > 0) {
+        if (workspace == nullptr ||
+            workspace_bytes < workspace_bytes_for(bh, split_heads, a.Dh, plan.n_splits))
             return FFA_ERR_WORKSPACE;
         if (!aligned16(workspace)) return FFA_ERR_ALIGNMENT;
         char* base = static_cast<char*>(workspace);
         ws.cnt = reinterpret_cast<unsigned int*>(base);
         ws.ml = reinterpret_cast<float*>(base + workspace_counter_bytes(bh));
-        ws.acc = reinterpret_cast<float*>(base + workspace_counter_bytes(bh) +
-                                          align_up((size_t)bh * plan.n_splits * 2 * sizeof(float), 256));
+        ws.acc = reinterpret_cast<float*>(
+            base + workspace_counter_bytes(bh) +
+            align_up((size_t)split_heads * plan.n_splits * 2 * sizeof(float), 256));
     }
     return launch_decode(a, plan, ws);
 }
@@ -115,7 +118,7 @@ int ffa_plan_launch(int precision, int batch_size, int head_num, int head_dim, i
 size_t ffa_workspace_bytes(int batch_size, int head_num, int head_dim, int max_seq_len) {
     if (batch_size <= 0 || head_num <= 0 || head_dim <= 0 || max_seq_len <= 0) return 0;
     const int bh = batch_size * head_num;
-    return workspace_bytes_for(bh, head_dim, max_splits_for(bh, max_seq_len));
+    return workspace_bytes_for(bh, bh, head_dim, max_splits_for(bh, max_seq_len));
 }
 
 int ffa_workspace_init(void* workspace, size_t workspace_bytes, void* stream) {

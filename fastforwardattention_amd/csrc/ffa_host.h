@@ -59,16 +59,17 @@ inline int max_splits_for(int bh, int max_seq_len) {
 
 inline size_t workspace_counter_bytes(int bh) { return align_up((size_t)bh * sizeof(unsigned int), 256); }
 
-inline size_t workspace_bytes_for(int bh, int head_dim, int n_splits) {
-    if (n_splits <= 1) return workspace_counter_bytes(bh);
-    return workspace_counter_bytes(bh) + align_up((size_t)bh * n_splits * 2 * sizeof(float), 256) +
-           (size_t)bh * n_splits * head_dim * sizeof(float);
+// bh = all (batch, head) pairs (counter array), split_heads = pairs that are split.
+inline size_t workspace_bytes_for(int bh, int split_heads, int head_dim, int n_splits) {
+    if (n_splits <= 1 || split_heads <= 0) return workspace_counter_bytes(bh);
+    return workspace_counter_bytes(bh) + align_up((size_t)split_heads * n_splits * 2 * sizeof(float), 256) +
+           (size_t)split_heads * n_splits * head_dim * sizeof(float);
 }
 
 // planner (ffa_plan.cpp)
 int plan_launch(int precision, int B, int H, int Dh, int t, float p, int use_default, int cus,
                 ffa_launch_plan* plan);
-int validate_plan(const ffa_launch_plan& plan, int precision, int t, float p);
+int validate_plan(const ffa_launch_plan& plan, int precision, int bh, int t, float p);
 
 // launchers (ffa_kernels.hip)
 int launch_decode(const DecodeArgs& a, const ffa_launch_plan& plan, const WorkspaceView& ws);

@@ -48,9 +48,38 @@ struct DecodeParams {
     float p;
     int right_or_no_padding;
     int n_splits, tiles_per_split;
+    int n_whole;  // (b,h) pairs [0, n_whole) get one workgroup each; the rest are split
     int bh_total;
     int combine;  // FFA_COMBINE_*
+#ifdef FFA_TRACE
+    unsigned long long* trace;  // [wave slot][16] timestamps, profiling builds only
+#endif
 };
+
+// Phase timestamps for profiling builds (-DFFA_TRACE): lane 0 of every wave stores the
+// 100 MHz wall clock into slot `s` of its row.  Compiles to nothing otherwise.
+#ifdef FFA_TRACE
+#define FFA_TP_ENTRY()                                                                         \
+    const unsigned long long ffa_t_entry = wall_clock64();                                     \
+    unsigned long long* ffa_row = nullptr;                                                     \
+    if (P.trace) {                                                                             \
+        const unsigned w = __builtin_amdgcn_readfirstlane(                                     \
+            blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6));                              \
+        ffa_row = P.trace + (size_t)w * 16;                                                    \
+        if ((threadIdx.x & 63) == 0) {                                                         \
+            ffa_row[9] = ffa_t_entry;                                                          \
+            ffa_row[8] = (unsigned long long)__builtin_amdgcn_s_getreg((31 << 11) | 4) |       \
+                         ((unsigned long long)__builtin_amdgcn_s_getreg((31 << 11) | 20) << 32); \
+        }                                                                                      \
+    }
+#define FFA_TP(s)                                                            \
+    do {                                                                     \
+        if (ffa_row && (threadIdx.x & 63) == 0) ffa_row[(s)] = wall_clock64(); \
+    } while (0)
+#else
+#define FFA_TP(s) do {} while (0)
+#define FFA_TP_ENTRY() do {} while (0)
+#endif
 
 // Per-(b) bounds, attention.cu:805-817.  tlen = slot of the new token = number of cached
 // keys; first = first unmasked key.  Values are clamped so that a bad seq_lengths entry
@@ -66,20 +95,54 @@ __device__ __forceinline__ void step_bounds(const DecodeParams& P, int b, int& t
 }
 
 // Append k_new, v_new at slot tlen of the (b,h) caches (attention.cu:901-914, :1246).
-// One wave: lanes < NCH move one 16-byte chunk of K and one of V each.
+// One wave: lane c < NCH moves 16-byte chunk c of K and of V (NCH <= 64).  The loads are
+// issued early (new_token_load) and the stores late (new_token_store), so that neither
+// round trip sits on the wave's critical path.
+struct NewToken {
+    uint4 k, v;
+};
 template <int NCH>
-__device__ __forceinline__ void append_new_token(char* kc_bh, char* vc_bh, const char* knew,
-                                                 const char* vnew, int tlen, int Lmax, int lane) {
-    for (int c = lane; c < NCH; c += kWave) {
-        st16(kc_bh + ((size_t)c * Lmax + tlen) * 16, ld16(knew + c * 16));
-        st16(vc_bh + ((size_t)tlen * NCH + c) * 16, ld16(vnew + c * 16));
+__device__ __forceinline__ NewToken new_token_load(const char* knew, const char* vnew, int lane) {
+    NewToken n;
+    const int c = lane < NCH ? lane : 0;
+    n.k = ld16(knew + c * 16);
+    n.v = ld16(vnew + c * 16);
+    return n;
+}
+template <int NCH>
+__device__ __forceinline__ void new_token_store(const NewToken& n, char* kc_bh, char* vc_bh, int tlen,
+                                                int Lmax, int lane) {
+    if (lane < NCH) {
+        st16(kc_bh + ((size_t)lane * Lmax + tlen) * 16, n.k);
+        st16(vc_bh + ((size_t)tlen * NCH + lane) * 16, n.v);
     }
 }
 
 // ---------------------------------------------------------------------------------------
 // One 64-key tile of q.K^T for the calling wave.  Lane l owns key tile*64+l; keys beyond
 // tlen read the new token's k (valid memory) and are masked by the caller.
-// Returns the raw dot product (not yet scaled).
+// load_k_group puts CG 16-byte loads in flight, dot_k_group consumes them.
+template <int CG>
+__device__ __forceinline__ void load_k_group(uint4 (&kv)[CG], const char* kp, size_t kstr, int g) {
+#pragma unroll
+    for (int c = 0; c < CG; ++c) kv[c] = ld16(kp + (size_t)(g * CG + c) * kstr);
+}
+
+template <typename T, int CG, bool Q_LDS>
+__device__ __forceinline__ float dot_k_group(const uint4 (&kv)[CG], int g, const uint4* q_reg,
+                                             const uint4* q_lds, float s) {
+#pragma unroll
+    for (int c = 0; c < CG; ++c) {
+        uint4 qc;
+        if constexpr (Q_LDS) qc = q_lds[g * CG + c];
+        else qc = q_reg[g * CG + c];
+        s = dot_chunk(kv[c], qc, s, T{});
+    }
+    return s;
+}
+
+// Whole-tile raw dot product (not yet scaled), NCH/CG groups, at most two groups of loads
+// in flight.
 template <typename T, int NCH, bool Q_LDS>
 __device__ __forceinline__ float tile_qk(const char* kc_bh, const char* knew, int key, int tlen,
                                          int Lmax, const uint4* q_reg, const uint4* q_lds) {
@@ -91,15 +154,8 @@ __device__ __forceinline__ float tile_qk(const char* kc_bh, const char* knew, in
 #pragma unroll 2
     for (int g = 0; g < NCH / CG; ++g) {
         uint4 kv[CG];
-#pragma unroll
-        for (int c = 0; c < CG; ++c) kv[c] = ld16(kp + (size_t)(g * CG + c) * kstr);
-#pragma unroll
-        for (int c = 0; c < CG; ++c) {
-            uint4 qc;
-            if constexpr (Q_LDS) qc = q_lds[g * CG + c];
-            else qc = q_reg[g * CG + c];
-            s = dot_chunk(kv[c], qc, s, T{});
-        }
+        load_k_group<CG>(kv, kp, kstr, g);
+        s = dot_k_group<T, CG, Q_LDS>(kv, g, q_reg, q_lds, s);
     }
     return s;
 }
@@ -110,7 +166,11 @@ struct Geo {
     static constexpr int NCH = DH / X;        // 16-byte chunks per key / per V row
     static constexpr int LPR = NCH;           // lanes per V row
     static constexpr int RPI = kWave / LPR;   // V rows per load instruction
+#ifdef FFA_Q_LDS_ALL
+    static constexpr bool Q_LDS = true;
+#else
     static constexpr bool Q_LDS = NCH > 16;   // q kept in LDS when it would not fit SGPR/VGPRs
+#endif
     static constexpr int QREG = Q_LDS ? 1 : NCH;
     static_assert(NCH >= 1 && NCH <= kWave && kWave % NCH == 0, "unsupported head dim");
 };
@@ -143,13 +203,24 @@ __global__ void __launch_bounds__(NW * 64) ffa_decode_split_kernel(const DecodeP
     __shared__ int s_last;
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    FFA_TP_ENTRY();
+    FFA_TP(0);
 
-    // Workgroups are handed to the 8 XCDs round-robin by index; keep every split of one
-    // (b,h) on one XCD so that partials are merged out of the L2 they were written to.
-    const int xcd = blockIdx.x & 7, r = blockIdx.x >> 3;
-    const int split = r % P.n_splits;
-    const int bh = (r / P.n_splits) * 8 + xcd;
-    if (bh >= P.bh_total) return;
+    // Work mapping.  The first n_whole workgroups each own a whole (b,h) pair and finish with
+    // an LDS merge only; the remaining pairs are cut into n_splits pieces whose partials are
+    // merged by the last piece to arrive.  Whole pairs are what the kernel ends on, so the
+    // cross-workgroup merges (a chain of memory round trips) finish in their shadow.
+    int bh, split, n_splits;
+    if ((int)blockIdx.x < P.n_whole) {
+        bh = blockIdx.x;
+        split = 0;
+        n_splits = 1;
+    } else {
+        const int r = blockIdx.x - P.n_whole;
+        bh = P.n_whole + r / P.n_splits;
+        split = r % P.n_splits;
+        n_splits = P.n_splits;
+    }
     const int b = bh / P.H;
 
     int tlen, first;
@@ -173,13 +244,14 @@ __global__ void __launch_bounds__(NW * 64) ffa_decode_split_kernel(const DecodeP
     }
 
     const int ntiles = tlen / kWave + 1;  // keys 0..tlen
-    const int tile_lo = max(split * P.tiles_per_split, first / kWave);
-    const int tile_hi = min(ntiles, (split + 1) * P.tiles_per_split);
-
-    // The workgroup owning the tile of slot tlen appends the new token.  Nobody reads
-    // slot tlen from the caches in this launch (it is always taken from k, v).
-    if (wave == 0 && split == min((ntiles - 1) / P.tiles_per_split, P.n_splits - 1))
-        append_new_token<NCH>(kc_bh, vc_bh, knew, vnew, tlen, P.Lmax, lane);
+    const int tps = n_splits == 1 ? ntiles : P.tiles_per_split;
+    const int tile_lo = max(split * tps, first / kWave);
+    const int tile_hi = min(ntiles, (split + 1) * tps);
+    // The workgroup owning the tile of slot tlen appends the new token (after its tile loop).
+    // Nobody reads slot tlen from the caches in this launch: it is always taken from k, v.
+    const bool appends = split == min((ntiles - 1) / tps, n_splits - 1) && wave == 0;
+    NewToken new_tok;
+    if (appends) new_tok = new_token_load<NCH>(knew, vnew, lane);
 
     const int rg = lane / LPR, dch = lane % LPR;
     float m_run = -INFINITY, l_run = 0.f;
@@ -197,12 +269,35 @@ __global__ void __launch_bounds__(NW * 64) ffa_decode_split_kernel(const DecodeP
         }
     };
 
-    for (int tile = tile_lo + wave; tile < tile_hi; tile += NW) {
+    constexpr int CG = NCH < 8 ? NCH : 8;
+
+    // First load groups of one tile: CG chunks of K (lane = key) and VG chunks of V
+    // (lane = row group x d-chunk).  V does not depend on the scores, so both go out together.
+    auto load_tile = [&](uint4 (&kv)[CG], uint4 (&vv)[VG], int tile) {
         const int key = tile * kWave + lane;
-        float s = tile_qk<T, NCH, G::Q_LDS>(kc_bh, knew, key, tlen, P.Lmax, q_reg, s_q);
-        // The V loads do not depend on the scores: put the first group in flight now.
-        uint4 vv[VG];
+        const bool cached = key < tlen;
+        const char* kp = cached ? kc_bh + (size_t)key * 16 : knew;
+        const size_t kstr = cached ? (size_t)P.Lmax * 16 : 16;
+        load_k_group<CG>(kv, kp, kstr, 0);
         load_v_group(vv, tile, 0);
+    };
+
+    // Scores, online softmax and P.V of one tile whose first load groups are in kv / vv.
+    auto compute_tile = [&](uint4 (&kv)[CG], uint4 (&vv)[VG], int tile) {
+        const int key = tile * kWave + lane;
+        float s = dot_k_group<T, CG, G::Q_LDS>(kv, 0, q_reg, s_q, 0.f);
+        if constexpr (NCH > CG) {
+            const bool cached = key < tlen;
+            const char* kp = cached ? kc_bh + (size_t)key * 16 : knew;
+            const size_t kstr = cached ? (size_t)P.Lmax * 16 : 16;
+#pragma unroll 2
+            for (int g = 1; g < NCH / CG; ++g) {
+                uint4 kn[CG];
+                load_k_group<CG>(kn, kp, kstr, g);
+                s = dot_k_group<T, CG, G::Q_LDS>(kn, g, q_reg, s_q, s);
+            }
+        }
+        FFA_TP(1);
 
         const bool valid = key <= tlen && key >= first;
         const float m_new = fmaxf(m_run, wave_max(valid ? s * P.scale_log2e : -INFINITY));
@@ -221,6 +316,7 @@ __global__ void __launch_bounds__(NW * 64) ffa_decode_split_kernel(const DecodeP
 #pragma unroll
         for (int e = 0; e < X; ++e) acc[e] *= alpha;
 
+        FFA_TP(2);
         const float* pst = &s_p[wave][rg * NCH];
 #pragma unroll
         for (int g = 0; g < NCH / VG; ++g) {
@@ -234,8 +330,40 @@ __global__ void __launch_bounds__(NW * 64) ffa_decode_split_kernel(const DecodeP
             }
         }
         __builtin_amdgcn_wave_barrier();
-    }
+    };
 
+    // The scheduling barrier keeps the compiler from sinking loads next to their uses to
+    // save registers, which would serialise the round trips.
+    for (int tile = tile_lo + wave; tile < tile_hi; tile += NW) {
+        uint4 kv[CG], vv[VG];
+        load_tile(kv, vv, tile);
+        __builtin_amdgcn_sched_barrier(0);
+#if !defined(FFA_ABL) || FFA_ABL != 2
+        compute_tile(kv, vv, tile);
+#else
+        acc[0] += __uint_as_float(kv[0].x ^ kv[7].y ^ vv[0].x ^ vv[7].w);
+#endif
+    }
+#if defined(FFA_ABL) && FFA_ABL == 1
+    if (acc[0] == 1.2345f) P.ws_ml[0] = acc[1] + l_run + m_run;
+    return;
+#endif
+
+#if !defined(FFA_ABL) || (FFA_ABL != 3 && FFA_ABL != 5)
+    if (appends) new_token_store<NCH>(new_tok, kc_bh, vc_bh, tlen, P.Lmax, lane);
+#endif
+#if defined(FFA_ABL) && FFA_ABL == 5
+    // timing experiment: only write-through (device-scope) stores leave the kernel
+    if (lane < 8) publish(&P.ws_ml[(size_t)bh * 8 + lane], acc[lane & 7] + l_run + m_run);
+    return;
+#endif
+#if defined(FFA_ABL) && FFA_ABL == 4
+    // timing experiment: no cross-wave merge, every wave stores something and leaves
+    if (lane < 8) reinterpret_cast<T*>(P.out)[(size_t)bh * DH + lane] = (T)(acc[lane & 7] + l_run + m_run);
+    return;
+#endif
+
+    FFA_TP(3);
     // ---- merge the waves of this workgroup (LDS) ----
     l_run = wave_sum(l_run);
     if (lane == 0) { s_m[wave] = m_run; s_l[wave] = l_run; }
@@ -255,7 +383,9 @@ __global__ void __launch_bounds__(NW * 64) ffa_decode_split_kernel(const DecodeP
     }
 
     T* out = reinterpret_cast<T*>(P.out) + (size_t)bh * DH;
-    float* wa = P.ws_acc + ((size_t)bh * P.n_splits + split) * DH;
+    // Partials of split pairs: slot (bh - n_whole) of the workspace.
+    const size_t slot0 = (size_t)(bh - P.n_whole) * P.n_splits;
+    float* wa = P.ws_acc + (slot0 + split) * DH;
     for (int d = tid; d < DH; d += NW * 64) {
         float o = 0.f;
 #pragma unroll
@@ -265,15 +395,15 @@ __global__ void __launch_bounds__(NW * 64) ffa_decode_split_kernel(const DecodeP
             for (int g = 0; g < RPI; ++g) ow += s_acc[w][g * DH + d];
             o += wgt[w] * ow;
         }
-        if (P.n_splits == 1) store_out(out, d, L > 0.f ? o / L : 0.f);
+        if (n_splits == 1) store_out(out, d, L > 0.f ? o / L : 0.f);
         else if (P.combine == FFA_COMBINE_FUSED) publish(&wa[d], o);
         else wa[d] = o;
     }
-    if (P.n_splits == 1) return;
+    if (n_splits == 1) return;
     if (P.combine != FFA_COMBINE_FUSED) {
         // A second kernel merges: plain stores would do, the kernel boundary publishes them.
         if (tid == 0) {
-            float* ml = P.ws_ml + ((size_t)bh * P.n_splits + split) * 2;
+            float* ml = P.ws_ml + (slot0 + split) * 2;
             ml[0] = M;
             ml[1] = L;
         }
@@ -289,41 +419,67 @@ __global__ void __launch_bounds__(NW * 64) ffa_decode_split_kernel(const DecodeP
     // outstanding memory operations), the arrival counter is bumped after it, and the
     // merging workgroup reads the partials only after it has seen the final count.
     if (tid == 0) {
-        float* ml = P.ws_ml + ((size_t)bh * P.n_splits + split) * 2;
+        float* ml = P.ws_ml + (slot0 + split) * 2;
         publish(&ml[0], M);
         publish(&ml[1], L);
     }
+    FFA_TP(4);
     __syncthreads();
+    FFA_TP(5);
     if (tid == 0) {
         const unsigned prev =
             __hip_atomic_fetch_add(&P.ws_cnt[bh], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        s_last = (prev == (unsigned)(P.n_splits - 1));
+        s_last = (prev == (unsigned)(n_splits - 1));
     }
     __syncthreads();
+    FFA_TP(6);
     if (!s_last) return;
 
-    const float* ml = P.ws_ml + (size_t)bh * P.n_splits * 2;
-    float Mg = -INFINITY;
-    for (int s = 0; s < P.n_splits; ++s) Mg = fmaxf(Mg, acquire(&ml[2 * s]));
+    // Merge: all loads of a batch of splits are issued before any is consumed.
+    const float* ml = P.ws_ml + slot0 * 2;
+    constexpr int MB = 8;
     for (int d = tid; d < DH; d += NW * 64) {
-        float o = 0.f, Lg = 0.f;
-        for (int s = 0; s < P.n_splits; ++s) {
-            const float ms = acquire(&ml[2 * s]);
-            const float w = (ms == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(ms - Mg);
-            Lg += w * acquire(&ml[2 * s + 1]);
-            o += w * acquire(&P.ws_acc[((size_t)bh * P.n_splits + s) * DH + d]);
+        float Mg = -INFINITY, o = 0.f, Lg = 0.f;
+        for (int s0 = 0; s0 < n_splits; s0 += MB) {
+            float ms[MB], ls[MB], as[MB];
+#pragma unroll
+            for (int j = 0; j < MB; ++j) {
+                const int sj = min(s0 + j, n_splits - 1);
+                ms[j] = acquire(&ml[2 * sj]);
+                ls[j] = acquire(&ml[2 * sj + 1]);
+                as[j] = acquire(&P.ws_acc[(slot0 + sj) * DH + d]);
+            }
+            float Mb = Mg;
+#pragma unroll
+            for (int j = 0; j < MB; ++j)
+                if (s0 + j < n_splits) Mb = fmaxf(Mb, ms[j]);
+            const float rescale = (Mg == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(Mg - Mb);
+            o *= rescale;
+            Lg *= rescale;
+#pragma unroll
+            for (int j = 0; j < MB; ++j) {
+                if (s0 + j < n_splits && ms[j] != -INFINITY) {
+                    const float w = __builtin_amdgcn_exp2f(ms[j] - Mb);
+                    Lg += w * ls[j];
+                    o += w * as[j];
+                }
+            }
+            Mg = Mb;
         }
         store_out(out, d, Lg > 0.f ? o / Lg : 0.f);
     }
+    FFA_TP(7);
     // Ready for the next launch on this stream (kernel boundaries order this store).
     if (tid == 0) __hip_atomic_store(&P.ws_cnt[bh], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
-// Merge kernel of FFA_COMBINE_KERNEL: one wave per (b,h), log-sum-exp over the splits.
+// Merge kernel of FFA_COMBINE_KERNEL: one wave per split (b,h) pair, log-sum-exp over its
+// partials.
 template <typename T, int DH>
 __global__ void __launch_bounds__(64) ffa_merge_splits_kernel(const DecodeParams P) {
-    const int bh = blockIdx.x, tid = threadIdx.x;
-    const float* ml = P.ws_ml + (size_t)bh * P.n_splits * 2;
+    const int bh = P.n_whole + blockIdx.x, tid = threadIdx.x;
+    const size_t slot0 = (size_t)blockIdx.x * P.n_splits;
+    const float* ml = P.ws_ml + slot0 * 2;
     float Mg = -INFINITY;
     for (int s = 0; s < P.n_splits; ++s) Mg = fmaxf(Mg, ml[2 * s]);
     T* out = reinterpret_cast<T*>(P.out) + (size_t)bh * DH;
@@ -333,7 +489,7 @@ __global__ void __launch_bounds__(64) ffa_merge_splits_kernel(const DecodeParams
             const float ms = ml[2 * s];
             const float w = (ms == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(ms - Mg);
             Lg += w * ml[2 * s + 1];
-            o += w * P.ws_acc[((size_t)bh * P.n_splits + s) * DH + d];
+            o += w * P.ws_acc[(slot0 + s) * DH + d];
         }
         store_out(out, d, Lg > 0.f ? o / Lg : 0.f);
     }
@@ -383,7 +539,8 @@ __global__ void __launch_bounds__(NW * 64) ffa_decode_wg_kernel(const DecodePara
     const int tile_lo = min(first / kWave, ntiles);  // tiles below are fully masked
     const bool pruned = P.p > 0.f;
 
-    if (wave == 0) append_new_token<NCH>(kc_bh, vc_bh, knew, vnew, tlen, P.Lmax, lane);
+    NewToken new_tok;
+    if (wave == 0) new_tok = new_token_load<NCH>(knew, vnew, lane);
 
     // ---- phase 1: raw scores to LDS, running max (exp2 domain) ----
     float mx = -INFINITY;
@@ -394,6 +551,7 @@ __global__ void __launch_bounds__(NW * 64) ffa_decode_wg_kernel(const DecodePara
         s_sc[key] = valid ? s : -INFINITY;  // raw dot product; scaled inside the exp2 below
         mx = fmaxf(mx, valid ? s * P.scale_log2e : -INFINITY);
     }
+    if (wave == 0) new_token_store<NCH>(new_tok, kc_bh, vc_bh, tlen, P.Lmax, lane);
     mx = wave_max(mx);
     if (lane == 0) s_red[wave] = mx;
     __syncthreads();
@@ -554,11 +712,11 @@ static int check_launch() {
 
 template <typename T, int DH, int NW>
 static int launch_split(const DecodeParams& P, hipStream_t st) {
-    const int groups = (P.bh_total + 7) / 8;
-    const dim3 grid((unsigned)(groups * 8 * P.n_splits));
+    const int n_split_heads = P.bh_total - P.n_whole;
+    const dim3 grid((unsigned)(P.n_whole + n_split_heads * P.n_splits));
     hipLaunchKernelGGL((ffa_decode_split_kernel<T, DH, NW>), grid, dim3(NW * 64), 0, st, P);
-    if (P.n_splits > 1 && P.combine == FFA_COMBINE_KERNEL)
-        hipLaunchKernelGGL((ffa_merge_splits_kernel<T, DH>), dim3((unsigned)P.bh_total), dim3(64), 0, st, P);
+    if (n_split_heads > 0 && P.n_splits > 1 && P.combine == FFA_COMBINE_KERNEL)
+        hipLaunchKernelGGL((ffa_merge_splits_kernel<T, DH>), dim3((unsigned)n_split_heads), dim3(64), 0, st, P);
     return check_launch();
 }
 
@@ -615,6 +773,11 @@ static int dispatch_head_dim(const DecodeParams& P, int head_dim, const ffa_laun
     }
 }
 
+#ifdef FFA_TRACE
+static unsigned long long* g_trace = nullptr;
+extern "C" void ffa_debug_set_trace(void* p) { g_trace = static_cast<unsigned long long*>(p); }
+#endif
+
 int launch_decode(const DecodeArgs& a, const ffa_launch_plan& plan, const WorkspaceView& ws) {
     DecodeParams P;
     P.q = a.q; P.k = a.k; P.v = a.v;
@@ -627,8 +790,12 @@ int launch_decode(const DecodeArgs& a, const ffa_launch_plan& plan, const Worksp
     P.p = a.p;
     P.right_or_no_padding = a.right_or_no_padding;
     P.n_splits = plan.n_splits; P.tiles_per_split = plan.tiles_per_split;
+    P.n_whole = plan.kind == FFA_LAUNCH_SPLIT ? plan.whole_heads : 0;
     P.bh_total = a.B * a.H;
     P.combine = plan.combine;
+#ifdef FFA_TRACE
+    P.trace = g_trace;
+#endif
     hipStream_t st = reinterpret_cast<hipStream_t>(a.stream);
     if (a.precision == FFA_PRECISION_F16) return dispatch_head_dim<uint16_t>(P, a.Dh, plan, st);
     return dispatch_head_dim<float>(P, a.Dh, plan, st);

@@ -28,7 +28,7 @@ static void fill(ffa_launch_plan* plan, int kind, int waves, int n_splits, int t
     plan->n_splits = n_splits;
     plan->tiles_per_split = tiles_per_split;
     plan->combine = FFA_COMBINE_FUSED;
-    plan->reserved = 0;
+    plan->whole_heads = 0;
 }
 
 // Largest power-of-two wave count (<= 16) whose score buffer + merge buffer fit in LDS and
@@ -71,21 +71,37 @@ int plan_launch(int precision, int B, int H, int Dh, int t, float p, int use_def
         return FFA_OK;
     }
 
-    // Exact path: split the sequence so that the launch has about `target` workgroups.
-    const int waves = wg_waves_for(ntiles, 4);
-    const int target = 6 * cus;
-    int n_splits = target / bh;
-    const int cap = max_splits_for(bh, (t + 1));
+    // Exact path.  With at least one (batch, head) pair per CU, give whole pairs to
+    // single workgroups in multiples of the CU count (every CU gets the same number, and
+    // the kernel ends on LDS-only merges) and split only the remainder, finely enough that
+    // its pieces also spread over all CUs and finish, merges included, long before the
+    // whole pairs do.  With fewer pairs than CUs everything is split.
+    int whole = (bh / cus) * cus;
+    const int rest = bh - whole;
+    int waves, n_splits = 1, tps = ntiles;
+    if (whole > 0) {
+        waves = wg_waves_for(ntiles, 4);
+        if (rest > 0) {
+            n_splits = ceil_div(cus, rest);
+            if (n_splits > ntiles) n_splits = ntiles;
+        }
+    } else {
+        waves = wg_waves_for(ntiles, 4);
+        n_splits = ceil_div(6 * cus, bh);
+        if (n_splits > ceil_div(ntiles, waves)) n_splits = ceil_div(ntiles, waves);
+    }
+    const int cap = max_splits_for(rest > 0 ? rest : bh, t + 1);
     if (n_splits > cap) n_splits = cap;
-    if (n_splits > ceil_div(ntiles, waves)) n_splits = ceil_div(ntiles, waves);
     if (n_splits < 1) n_splits = 1;
-    const int tps = ceil_div(ntiles, n_splits);
+    tps = ceil_div(ntiles, n_splits);
     n_splits = ceil_div(ntiles, tps);
+    if (n_splits == 1) whole = bh;  // nothing left to split: plain one-workgroup-per-pair
     fill(plan, FFA_LAUNCH_SPLIT, waves, n_splits, tps);
+    plan->whole_heads = whole;
     return FFA_OK;
 }
 
-int validate_plan(const ffa_launch_plan& plan, int precision, int t, float p) {
+int validate_plan(const ffa_launch_plan& plan, int precision, int bh, int t, float p) {
     const int w = plan.waves_per_wg;
     if (w != 1 && w != 2 && w != 4 && w != 8 && w != 16) return FFA_ERR_PLAN;
     if (plan.threads_per_key != 1 || plan.keys_per_wave != kTileKeys) return FFA_ERR_PLAN;
@@ -94,14 +110,18 @@ int validate_plan(const ffa_launch_plan& plan, int precision, int t, float p) {
     const int ntiles = num_tiles(t);
     switch (plan.kind) {
         case FFA_LAUNCH_WORKGROUP:
-            if (plan.n_splits != 1) return FFA_ERR_PLAN;
+            if (plan.n_splits != 1 || plan.whole_heads != 0) return FFA_ERR_PLAN;
             if (wg_dynamic_lds_bytes(t, w, precision / 8) > (size_t)kMaxDynamicLdsBytes)
                 return FFA_ERR_TOO_LONG;
             return FFA_OK;
         case FFA_LAUNCH_SPLIT:
             if (p > 0.f) return FFA_ERR_PLAN;  // the split kernel is the exact path only
             if (w > 8) return FFA_ERR_PLAN;
-            if ((long long)plan.n_splits * plan.tiles_per_split < ntiles) return FFA_ERR_PLAN;
+            if (plan.whole_heads < 0 || plan.whole_heads > bh) return FFA_ERR_PLAN;
+            if (plan.whole_heads < bh && (long long)plan.n_splits * plan.tiles_per_split < ntiles)
+                return FFA_ERR_PLAN;
+            if ((long long)(bh - plan.whole_heads) * plan.n_splits > 4 * kMaxSplitWorkgroups)
+                return FFA_ERR_PLAN;
             return FFA_OK;
         default:
             return FFA_ERR_PLAN;

@@ -152,7 +152,8 @@ struct FastForwardAttn {
     }
 
     // Not in the reference: the plan the next call at (t, p) would use, as
-    // (kind, waves_per_wg, threads_per_key, keys_per_wave, n_splits, tiles_per_split, combine).
+    // (kind, waves_per_wg, threads_per_key, keys_per_wave, n_splits, tiles_per_split, combine,
+    //  whole_heads).
     std::vector<int> launch_plan(int curr_timestep, float prob_thresh) {
         const CacheDims d = dims_of(k_cache, v_cache);
         ffa_launch_plan plan;
@@ -160,7 +161,7 @@ struct FastForwardAttn {
                                      ft_kernel_launch ? 1 : 0, 0, &plan),
                      "launch planning");
         return {plan.kind, plan.waves_per_wg, plan.threads_per_key, plan.keys_per_wave, plan.n_splits,
-                plan.tiles_per_split, plan.combine};
+                plan.tiles_per_split, plan.combine, plan.whole_heads};
     }
 
     torch::Tensor k_cache;

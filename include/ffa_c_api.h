@@ -56,8 +56,9 @@ typedef enum ffa_status {
 /* Launch kinds. */
 #define FFA_LAUNCH_WORKGROUP 0  /* one workgroup per (batch, head); scores staged in LDS;   */
                                 /* any p >= 0.  The analogue of the reference's launch.     */
-#define FFA_LAUNCH_SPLIT 1      /* sequence split over n_splits workgroups per (batch,      */
-                                /* head), online softmax, last-arriver combine; p == 0 only */
+#define FFA_LAUNCH_SPLIT 1      /* online-softmax kernel, p == 0 only: whole_heads pairs    */
+                                /* with one workgroup each, the others split over n_splits  */
+                                /* workgroups whose partials the last arriver combines      */
 
 /* How the partial (max, sum, acc[Dh]) results of a split launch are merged. */
 #define FFA_COMBINE_FUSED 0     /* by the last workgroup of each (batch, head) to arrive     */
@@ -72,7 +73,9 @@ typedef struct ffa_launch_plan {
     int32_t n_splits;         /* workgroups per (batch, head); 1 for FFA_LAUNCH_WORKGROUP  */
     int32_t tiles_per_split;  /* 64-key tiles each split walks                             */
     int32_t combine;          /* FFA_COMBINE_*: how split partials are merged              */
-    int32_t reserved;
+    int32_t whole_heads;      /* FFA_LAUNCH_SPLIT: the first whole_heads (batch, head)     */
+                              /* pairs get ONE workgroup each (no cross-workgroup merge);  */
+                              /* only the remaining pairs are split n_splits ways          */
 } ffa_launch_plan;
 
 int ffa_api_version(void);

@@ -117,4 +117,4 @@ def test_pruned_diag_and_stream():
         o2 = ffa.attention(q, k, v, 0.5, L, 0)
     s.synchronize()
     assert torch.equal(o2, exact)
-    assert len(ffa.launch_plan(L, 0.0)) == 7
+    assert len(ffa.launch_plan(L, 0.0)) == 8

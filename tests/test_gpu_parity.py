@@ -40,6 +40,16 @@ def _plans(prec, B, H, Dh, t):
             plans.append((f"split_w{waves}_tps{tps}", capi.make_plan(capi.FFA_LAUNCH_SPLIT, waves, ns, tps)))
             plans.append((f"split_w{waves}_tps{tps}_mergekernel",
                           capi.make_plan(capi.FFA_LAUNCH_SPLIT, waves, ns, tps, capi.FFA_COMBINE_KERNEL)))
+    # hybrid launches: some (batch, head) pairs whole, the rest split
+    bh = B * H
+    for whole in sorted({1, bh // 2, bh - 1, bh}):
+        if 0 < whole <= bh:
+            tps = max(1, ntiles // 3)
+            ns = -(-ntiles // tps)
+            plans.append((f"hybrid_whole{whole}_w8_tps{tps}",
+                          capi.make_plan(capi.FFA_LAUNCH_SPLIT, 8, ns, tps, capi.FFA_COMBINE_FUSED, whole)))
+            plans.append((f"hybrid_whole{whole}_w2_tps{tps}_mergekernel",
+                          capi.make_plan(capi.FFA_LAUNCH_SPLIT, 2, ns, tps, capi.FFA_COMBINE_KERNEL, whole)))
     return plans
 
 

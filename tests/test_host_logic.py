@@ -77,6 +77,9 @@ def test_attention_argument_validation(lib):
     assert _attn(lib, plan=capi.make_plan(capi.FFA_LAUNCH_WORKGROUP, 4, 2, 1)) == 8
     assert _attn(lib, plan=capi.make_plan(7, 4, 1, 1)) == 8
     assert _attn(lib, plan=capi.make_plan(capi.FFA_LAUNCH_SPLIT, 4, 1, 1, combine=5)) == 8
+    assert _attn(lib, plan=capi.make_plan(capi.FFA_LAUNCH_SPLIT, 4, 1, 1, whole_heads=9)) == 8   # B*H = 8
+    assert _attn(lib, plan=capi.make_plan(capi.FFA_LAUNCH_SPLIT, 4, 1, 1, whole_heads=-1)) == 8
+    assert _attn(lib, plan=capi.make_plan(capi.FFA_LAUNCH_WORKGROUP, 4, 1, 1, whole_heads=2)) == 8
     assert _attn(lib, t=100, plan=capi.make_plan(capi.FFA_LAUNCH_SPLIT, 4, 1, 1)) == 8   # 1 tile < 2 needed
     assert _attn(lib, p=0.1, plan=capi.make_plan(capi.FFA_LAUNCH_SPLIT, 4, 2, 1)) == 8   # split is exact only
     assert _attn(lib, plan=capi.make_plan(capi.FFA_LAUNCH_SPLIT, 16, 2, 1)) == 8
@@ -109,9 +112,10 @@ def test_workspace_bytes_covers_every_plan(lib):
                 for cus in (64, 256, 304):
                     plan = capi.plan_launch(prec, B, H, Dh, t, 0.0, False, cus)
                     bh = B * H
+                    sh = bh - plan.whole_heads
                     need = -(-bh * 4 // 256) * 256
-                    if plan.n_splits > 1:
-                        need += -(-bh * plan.n_splits * 8 // 256) * 256 + bh * plan.n_splits * Dh * 4
+                    if plan.n_splits > 1 and sh > 0:
+                        need += -(-sh * plan.n_splits * 8 // 256) * 256 + sh * plan.n_splits * Dh * 4
                     assert need <= total, (B, H, Dh, Lmax, t, plan)
     assert lib.ffa_workspace_bytes(0, 1, 64, 8) == 0
 
@@ -133,8 +137,12 @@ def test_planner_consistency(prec, Dh):
                     else:
                         assert plan.kind == capi.FFA_LAUNCH_SPLIT
                         assert (plan.n_splits - 1) * plan.tiles_per_split < ntiles  # no empty split
-                        assert B * H * plan.n_splits <= 16384
+                        assert 0 <= plan.whole_heads <= B * H
+                        assert plan.whole_heads % 256 == 0 or plan.whole_heads == B * H
+                        assert (B * H - plan.whole_heads) * plan.n_splits <= 16384
                         assert plan.waves_per_wg <= 8
+                        if plan.n_splits == 1:
+                            assert plan.whole_heads == B * H
 
 
 def test_planner_default_follows_length_table():
