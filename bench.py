@@ -231,14 +231,141 @@ def cpu_baseline(wl, budget_s=15.0, max_steps=64):
     }
 
 
-def load_traffic(name):
-    """HBM bytes per launch measured with rocprofv3 --pmc (FETCH_SIZE, WRITE_SIZE), kept in
-    profiles/traffic.json by hand after a counter run; None when not measured."""
+class PrunedWorkload:
+    """BASELINE.json configs[4]: B=16, 32x64, fp16, 8192 cached keys, 64 decode steps,
+    peaked keys: per head 32 random positions hold 4*q_dir + N(0, 0.1), the rest N(0,1);
+    V is N(0,1).  The query is held fixed per head over the 64 steps (the peaks are built
+    for it once); k and v of the new token are fresh N(0,1) draws."""
+
+    def __init__(self, B=16, H=32, Dh=64, L=8192, gen=64):
+        import torch
+        from fastforwardattention_amd import capi
+        self.torch, self.capi, self.lib = torch, capi, capi.load()
+        self.B, self.H, self.Dh, self.L, self.gen, self.Lmax = B, H, Dh, L, gen, L + gen
+        self.scale = 0.125
+        dev = "cuda:0"
+        g = torch.Generator(device=dev).manual_seed(0)
+        q = torch.randn(B, H, Dh, device=dev, generator=g)
+        qdir = q / q.norm(dim=-1, keepdim=True)
+        K = torch.randn(B, H, L, Dh, device=dev, generator=g)
+        pos = torch.rand(B, H, L, device=dev, generator=g).argsort(dim=-1)[:, :, :32]      # 32 distinct positions
+        peaks = 4 * qdir[:, :, None, :] + 0.1 * torch.randn(B, H, 32, Dh, device=dev, generator=g)
+        K.scatter_(2, pos[..., None].expand(-1, -1, -1, Dh), peaks)
+        K = K.half()
+        V = torch.randn(B, H, L, Dh, device=dev, generator=g).half()
+        self.kc = torch.empty(B, H, Dh // 8, self.Lmax, 8, dtype=torch.float16, device=dev)
+        self.vc = torch.empty(B, H, self.Lmax, Dh, dtype=torch.float16, device=dev)
+        capi.check(self.lib.ffa_init_cache_f16(self.kc.data_ptr(), self.vc.data_ptr(), K.data_ptr(), V.data_ptr(),
+                                               B, L, self.Lmax, Dh, H, None), "ffa_init_cache_f16")
+        torch.cuda.synchronize()
+        del K, V
+        self.q = q.half()
+        self.k = torch.randn(gen, B, H, Dh, device=dev, generator=g).half()
+        self.v = torch.randn(gen, B, H, Dh, device=dev, generator=g).half()
+        self.out = torch.empty(gen, B, H, Dh, dtype=torch.float16, device=dev)
+        nbytes = self.lib.ffa_workspace_bytes(B, H, Dh, self.Lmax)
+        self.ws = torch.zeros(nbytes, dtype=torch.uint8, device=dev)
+        self.kept = torch.zeros(B, H, dtype=torch.int32, device=dev)
+        torch.cuda.synchronize()
+
+    def launch(self, i, p, stream_ptr, diag=False):
+        t = self.L + i % self.gen
+        plan = self.capi.plan_launch(16, self.B, self.H, self.Dh, t, p, False, self.lib.ffa_device_compute_units())
+        rc = self.lib.ffa_attention_diag(
+            16, self.B, self.H, self.Dh, self.Lmax, self.scale, t, self.q.data_ptr(),
+            self.k[i % self.gen].data_ptr(), self.v[i % self.gen].data_ptr(), self.kc.data_ptr(),
+            self.vc.data_ptr(), self.out[i % self.gen].data_ptr(), None, p,
+            None if diag else C.byref(plan), 1, self.ws.data_ptr(), self.ws.numel(),
+            self.kept.data_ptr() if diag else None, None, stream_ptr)
+        if rc != 0:
+            raise RuntimeError(f"ffa_attention_diag failed: {self.capi.status_string(rc)}")
+        return plan
+
+    def run(self, p, steps=64, warmup=8):
+        torch = self.torch
+        sp = torch.cuda.current_stream().cuda_stream
+        for i in range(warmup):
+            plan = self.launch(i, p, sp)
+
+        def body():
+            for i in range(steps):
+                self.launch(i, p, sp)
+        ms = time_region(torch, body)
+        out_p = self.out.clone()
+        # skip fraction at the last step (diagnostic launch, untimed)
+        self.launch(steps - 1, p, sp, diag=True)
+        torch.cuda.synchronize()
+        t_last = self.L + (steps - 1) % self.gen
+        skip_frac = 1.0 - float(self.kept.sum().item()) / (self.B * self.H * t_last)
+        return ms * 1e3 / steps, skip_frac, out_p, plan
+
+
+def run_pruned_sweep():
+    wl = PrunedWorkload()
+    res = []
+    ref = None
+    bytes_full = sum(algorithmic_bytes(wl.B, wl.H, wl.Dh, wl.L + i) for i in range(wl.gen)) / wl.gen
+    for p in (0.0, 1e-4, 1e-3, 1e-2):
+        us, skip, out, plan = wl.run(p)
+        if ref is None:
+            ref = out
+        err = float((out.float() - ref.float()).abs().max().item())
+        actual = bytes_full * (1.0 - 0.5 * skip)
+        res.append({"p": p, "us_per_step": round(us, 2), "skip_fraction": round(skip, 5),
+                    "max_abs_vs_p0": err, "effective_GBps": round(bytes_full / us / 1e3, 1),
+                    "actual_GBps": round(actual / us / 1e3, 1), "plan": repr(plan)})
+    return {"workload": "pruned sweep: B=16 H=32 Dh=64 fp16, 8192 cached keys, 64 steps, 32 peaked keys/head, "
+                        "query fixed per head", "algorithmic_bytes_per_step": round(bytes_full), "results": res}
+
+
+def run_suite(args):
+    """Every BASELINE.json configuration that fits one GPU, one JSON object per line."""
+    for name in ["opt1.3b_b10", "opt1.3b_b5", "opt1.3b_b2", "opt1.3b_b1", "gptj_b8",
+                 "long_b1_1k", "long_b1_2k", "long_b1_4k", "long_b1_8k", "long_b1_16k"]:
+        for use_default in (False, True):
+            wl = Workload(name, use_default=use_default)
+            steps = wl.layers * min(wl.gen, 64)
+            ms = run_graph(wl, steps, wl.layers)
+            us = ms * 1e3 / steps
+            mb = wl.mean_bytes(steps)
+            print(json.dumps({"workload": name, "use_default_kernel_launch": use_default, "steps": steps,
+                              "t_range": [wl.t_of(0), wl.t_of(steps - 1)], "us_per_step": round(us, 2),
+                              "GBps": round(mb / us / 1e3, 1), "hbm_frac": round(mb / us / 1e3 / HBM_PEAK_GBS, 4),
+                              "plan": repr(wl.plan_for(wl.t_of(0)))}), flush=True)
+            del wl
+            import torch
+            torch.cuda.empty_cache()
+    print(json.dumps(run_pruned_sweep()), flush=True)
+
+
+def run_copy_calibration(mib=128, reps=40):
+    """A plain device-to-device copy kernel of known size, for scaling rocprofv3's
+    FETCH_SIZE / WRITE_SIZE readings: every launch reads `mib` MiB and writes `mib` MiB.
+    Rotates over enough buffers that the source is never cache-resident."""
+    import torch
+    n = mib * (1 << 20) // 4
+    nbuf = 6
+    src = [torch.full((n,), float(i + 1), dtype=torch.float32, device="cuda:0") for i in range(nbuf)]
+    dst = [torch.empty(n, dtype=torch.float32, device="cuda:0") for _ in range(nbuf)]
+    torch.cuda.synchronize()
+    for i in range(reps):
+        dst[i % nbuf].copy_(src[i % nbuf])
+    torch.cuda.synchronize()
+    print(json.dumps({"calibration": "torch elementwise copy kernel", "bytes_read_per_launch": mib << 20,
+                      "bytes_written_per_launch": mib << 20, "launches": reps}))
+
+
+def load_traffic(name, algorithmic_bytes):
+    """HBM bytes per launch: the ratio (FETCH_SIZE + WRITE_SIZE, each scaled by a plain copy
+    kernel of known size) / algorithmic bytes measured with rocprofv3 --pmc and recorded in
+    profiles/traffic.json, applied to this run's algorithmic mean.  None when the workload
+    has no counter run on record."""
     path = os.path.join(ROOT, "profiles", "traffic.json")
     try:
         with open(path) as f:
-            return json.load(f).get(name)
-    except (OSError, ValueError):
+            rec = json.load(f).get(name)
+        return round(rec["hbm_bytes_over_algorithmic_bytes"] * algorithmic_bytes) if rec else None
+    except (OSError, ValueError, KeyError):
         return None
 
 
@@ -252,6 +379,13 @@ def main():
     ap.add_argument("--plan", default=None, help="kind,waves,tiles_per_split[,combine[,whole_heads]] (kind: 0 workgroup, 1 split; combine: 0 fused, 1 kernel)")
     ap.add_argument("--legs", default="graph,capi,ext", help="comma list of graph,capi,ext")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--suite", action="store_true",
+                    help="run every BASELINE configuration (tuned and default launch) and the pruned sweep; "
+                         "one JSON line each instead of the single headline line")
+    ap.add_argument("--pruned-sweep", action="store_true", help="only the pruned sweep (BASELINE configs[4])")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="run a plain 128 MiB copy kernel 40 times (reference for rocprofv3 --pmc FETCH_SIZE / "
+                         "WRITE_SIZE scaling) and exit")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on exactly one GPU (one process, one MI355X); "
@@ -262,6 +396,16 @@ def main():
     if not torch.cuda.is_available():
         print("bench.py: no GPU visible; the hot path has no CPU fallback.", file=sys.stderr)
         sys.exit(3)
+
+    if args.calibrate_copy:
+        run_copy_calibration()
+        return
+    if args.suite:
+        run_suite(args)
+        return
+    if args.pruned_sweep:
+        print(json.dumps(run_pruned_sweep()))
+        return
 
     plan_override = tuple(int(x) for x in args.plan.split(",")) if args.plan else None
     wl = Workload(args.workload, use_default=args.default_launch, plan_override=plan_override)
@@ -298,7 +442,7 @@ def main():
                    "launch_plan_at_first_step": repr(plan0)},
         "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(gbs / HBM_PEAK_GBS, 4),
-                     "traffic": load_traffic(args.workload),
+                     "traffic": load_traffic(args.workload, mean_b),
                      "algorithmic_bytes_per_launch": round(mean_b),
                      "kernel": "ffa_decode_split_kernel" if plan0.kind == 1 else "ffa_decode_wg_kernel",
                      "launch_us": round(us_step, 3)},
