@@ -72,9 +72,11 @@ struct DecodeParams {
                          ((unsigned long long)__builtin_amdgcn_s_getreg((31 << 11) | 20) << 32); \
         }                                                                                      \
     }
+// FFA_TRACE=2 keeps only the points that cost no registers in the hot loop (3 and later).
 #define FFA_TP(s)                                                            \
     do {                                                                     \
-        if (ffa_row && (threadIdx.x & 63) == 0) ffa_row[(s)] = wall_clock64(); \
+        if ((FFA_TRACE < 2 || (s) >= 3) && ffa_row && (threadIdx.x & 63) == 0) \
+            ffa_row[(s)] = wall_clock64();                                    \
     } while (0)
 #else
 #define FFA_TP(s) do {} while (0)
@@ -166,11 +168,7 @@ struct Geo {
     static constexpr int NCH = DH / X;        // 16-byte chunks per key / per V row
     static constexpr int LPR = NCH;           // lanes per V row
     static constexpr int RPI = kWave / LPR;   // V rows per load instruction
-#ifdef FFA_Q_LDS_ALL
-    static constexpr bool Q_LDS = true;
-#else
     static constexpr bool Q_LDS = NCH > 16;   // q kept in LDS when it would not fit SGPR/VGPRs
-#endif
     static constexpr int QREG = Q_LDS ? 1 : NCH;
     static_assert(NCH >= 1 && NCH <= kWave && kWave % NCH == 0, "unsupported head dim");
 };
@@ -197,7 +195,7 @@ __global__ void __launch_bounds__(NW * 64) ffa_decode_split_kernel(const DecodeP
     constexpr int VG = NCH < 8 ? NCH : 8;  // V loads kept in flight per group
 
     __shared__ float s_p[NW][kWave];
-    __shared__ float s_acc[NW][kWave * X];
+    __shared__ float s_acc[NW][DH];
     __shared__ float s_m[NW], s_l[NW];
     __shared__ uint4 s_q[G::Q_LDS ? NCH : 1];
     __shared__ int s_last;
@@ -332,43 +330,30 @@ __global__ void __launch_bounds__(NW * 64) ffa_decode_split_kernel(const DecodeP
         __builtin_amdgcn_wave_barrier();
     };
 
-    // The scheduling barrier keeps the compiler from sinking loads next to their uses to
+    // The scheduling barriers keep the compiler from sinking loads next to their uses to
     // save registers, which would serialise the round trips.
     for (int tile = tile_lo + wave; tile < tile_hi; tile += NW) {
         uint4 kv[CG], vv[VG];
         load_tile(kv, vv, tile);
         __builtin_amdgcn_sched_barrier(0);
-#if !defined(FFA_ABL) || FFA_ABL != 2
         compute_tile(kv, vv, tile);
-#else
-        acc[0] += __uint_as_float(kv[0].x ^ kv[7].y ^ vv[0].x ^ vv[7].w);
-#endif
     }
-#if defined(FFA_ABL) && FFA_ABL == 1
-    if (acc[0] == 1.2345f) P.ws_ml[0] = acc[1] + l_run + m_run;
-    return;
-#endif
-
-#if !defined(FFA_ABL) || (FFA_ABL != 3 && FFA_ABL != 5)
     if (appends) new_token_store<NCH>(new_tok, kc_bh, vc_bh, tlen, P.Lmax, lane);
-#endif
-#if defined(FFA_ABL) && FFA_ABL == 5
-    // timing experiment: only write-through (device-scope) stores leave the kernel
-    if (lane < 8) publish(&P.ws_ml[(size_t)bh * 8 + lane], acc[lane & 7] + l_run + m_run);
-    return;
-#endif
-#if defined(FFA_ABL) && FFA_ABL == 4
-    // timing experiment: no cross-wave merge, every wave stores something and leaves
-    if (lane < 8) reinterpret_cast<T*>(P.out)[(size_t)bh * DH + lane] = (T)(acc[lane & 7] + l_run + m_run);
-    return;
-#endif
 
     FFA_TP(3);
-    // ---- merge the waves of this workgroup (LDS) ----
+    // ---- merge inside the wave: the RPI row groups (lanes with equal lane % LPR) ----
+#pragma unroll
+    for (int off = LPR; off < kWave; off <<= 1) {
+#pragma unroll
+        for (int e = 0; e < X; ++e) acc[e] += __shfl_xor(acc[e], off);
+    }
+    // ---- merge the waves of this workgroup (LDS): DH floats + (max, sum) per wave ----
     l_run = wave_sum(l_run);
     if (lane == 0) { s_m[wave] = m_run; s_l[wave] = l_run; }
+    if (lane < LPR) {
 #pragma unroll
-    for (int e = 0; e < X; ++e) s_acc[wave][lane * X + e] = acc[e];
+        for (int e = 0; e < X; ++e) s_acc[wave][lane * X + e] = acc[e];
+    }
     __syncthreads();
 
     float M = -INFINITY;
@@ -389,12 +374,7 @@ __global__ void __launch_bounds__(NW * 64) ffa_decode_split_kernel(const DecodeP
     for (int d = tid; d < DH; d += NW * 64) {
         float o = 0.f;
 #pragma unroll
-        for (int w = 0; w < NW; ++w) {
-            float ow = 0.f;
-#pragma unroll
-            for (int g = 0; g < RPI; ++g) ow += s_acc[w][g * DH + d];
-            o += wgt[w] * ow;
-        }
+        for (int w = 0; w < NW; ++w) o += wgt[w] * s_acc[w][d];
         if (n_splits == 1) store_out(out, d, L > 0.f ? o / L : 0.f);
         else if (P.combine == FFA_COMBINE_FUSED) publish(&wa[d], o);
         else wa[d] = o;

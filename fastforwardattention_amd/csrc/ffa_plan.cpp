@@ -71,29 +71,29 @@ int plan_launch(int precision, int B, int H, int Dh, int t, float p, int use_def
         return FFA_OK;
     }
 
-    // Exact path.  With at least one (batch, head) pair per CU, give whole pairs to
-    // single workgroups in multiples of the CU count (every CU gets the same number, and
-    // the kernel ends on LDS-only merges) and split only the remainder, finely enough that
-    // its pieces also spread over all CUs and finish, merges included, long before the
-    // whole pairs do.  With fewer pairs than CUs everything is split.
+    // Exact path.  Measured on MI355X: the launch runs best with about one 4-wave workgroup
+    // per CU, each walking a long run of tiles, and with as few cross-workgroup merges as
+    // possible at the END of the kernel (a merge is a chain of three HBM-latency hops).
+    //  - At least one (batch, head) pair per CU: whole pairs go to single workgroups in
+    //    multiples of the CU count (every CU gets the same number, LDS-only merge); only the
+    //    remainder is split, into ceil(CUs/rest) pieces per pair, so that the pieces also
+    //    cover all CUs and are done, merges included, long before the whole pairs are.
+    //  - Fewer pairs than CUs: floor(CUs/pairs) pieces per pair (one workgroup per CU), but
+    //    never so many that a wave is left without a tile.
+    const int waves = wg_waves_for(ntiles, 4);
     int whole = (bh / cus) * cus;
     const int rest = bh - whole;
-    int waves, n_splits = 1, tps = ntiles;
+    int n_splits = 1;
     if (whole > 0) {
-        waves = wg_waves_for(ntiles, 4);
-        if (rest > 0) {
-            n_splits = ceil_div(cus, rest);
-            if (n_splits > ntiles) n_splits = ntiles;
-        }
+        if (rest > 0) n_splits = ceil_div(cus, rest);
     } else {
-        waves = wg_waves_for(ntiles, 4);
-        n_splits = ceil_div(6 * cus, bh);
-        if (n_splits > ceil_div(ntiles, waves)) n_splits = ceil_div(ntiles, waves);
+        n_splits = cus / bh;
     }
+    if (n_splits > ceil_div(ntiles, waves)) n_splits = ceil_div(ntiles, waves);
     const int cap = max_splits_for(rest > 0 ? rest : bh, t + 1);
     if (n_splits > cap) n_splits = cap;
     if (n_splits < 1) n_splits = 1;
-    tps = ceil_div(ntiles, n_splits);
+    const int tps = ceil_div(ntiles, n_splits);
     n_splits = ceil_div(ntiles, tps);
     if (n_splits == 1) whole = bh;  // nothing left to split: plain one-workgroup-per-pair
     fill(plan, FFA_LAUNCH_SPLIT, waves, n_splits, tps);
