@@ -237,8 +237,9 @@ class PrunedWorkload:
     V is N(0,1).  The query is held fixed per head over the 64 steps (the peaks are built
     for it once); k and v of the new token are fresh N(0,1) draws."""
 
-    def __init__(self, B=16, H=32, Dh=64, L=8192, gen=64):
+    def __init__(self, B=16, H=32, Dh=64, L=8192, gen=64, kind="library"):
         import torch
+        self.kind = kind
         from fastforwardattention_amd import capi
         self.torch, self.capi, self.lib = torch, capi, capi.load()
         self.B, self.H, self.Dh, self.L, self.gen, self.Lmax = B, H, Dh, L, gen, L + gen
@@ -268,14 +269,27 @@ class PrunedWorkload:
         self.kept = torch.zeros(B, H, dtype=torch.int32, device=dev)
         torch.cuda.synchronize()
 
+    def plan_for(self, t, p):
+        capi = self.capi
+        cus = self.lib.ffa_device_compute_units()
+        if self.kind == "library":
+            return capi.plan_launch(16, self.B, self.H, self.Dh, t, p, False, cus)
+        ntiles = t // 64 + 1
+        if self.kind == "workgroup":
+            return capi.make_plan(capi.FFA_LAUNCH_WORKGROUP, 16, 1, ntiles)
+        n = max(1, min(cus // (self.B * self.H), ntiles // 4))      # "two_pass"
+        tps = -(-ntiles // n)
+        return capi.make_plan(capi.FFA_LAUNCH_TWO_PASS, 4, -(-ntiles // tps), tps)
+
     def launch(self, i, p, stream_ptr, diag=False):
         t = self.L + i % self.gen
-        plan = self.capi.plan_launch(16, self.B, self.H, self.Dh, t, p, False, self.lib.ffa_device_compute_units())
+        plan = self.plan_for(t, p)
         rc = self.lib.ffa_attention_diag(
             16, self.B, self.H, self.Dh, self.Lmax, self.scale, t, self.q.data_ptr(),
             self.k[i % self.gen].data_ptr(), self.v[i % self.gen].data_ptr(), self.kc.data_ptr(),
             self.vc.data_ptr(), self.out[i % self.gen].data_ptr(), None, p,
-            None if diag else C.byref(plan), 1, self.ws.data_ptr(), self.ws.numel(),
+            None if (diag and plan.kind == self.capi.FFA_LAUNCH_SPLIT) else C.byref(plan), 1,
+            self.ws.data_ptr(), self.ws.numel(),
             self.kept.data_ptr() if diag else None, None, stream_ptr)
         if rc != 0:
             raise RuntimeError(f"ffa_attention_diag failed: {self.capi.status_string(rc)}")
@@ -300,8 +314,10 @@ class PrunedWorkload:
         return ms * 1e3 / steps, skip_frac, out_p, plan
 
 
-def run_pruned_sweep():
-    wl = PrunedWorkload()
+def run_pruned_sweep(B=16, kind="library"):
+    """kind: "library" = the planner's choice; "workgroup" / "two_pass" force that launch kind
+    (p = 0 included, so the two pruning-capable paths can be compared like for like)."""
+    wl = PrunedWorkload(B=B, kind=kind)
     res = []
     ref = None
     bytes_full = sum(algorithmic_bytes(wl.B, wl.H, wl.Dh, wl.L + i) for i in range(wl.gen)) / wl.gen
@@ -314,8 +330,16 @@ def run_pruned_sweep():
         res.append({"p": p, "us_per_step": round(us, 2), "skip_fraction": round(skip, 5),
                     "max_abs_vs_p0": err, "effective_GBps": round(bytes_full / us / 1e3, 1),
                     "actual_GBps": round(actual / us / 1e3, 1), "plan": repr(plan)})
-    return {"workload": "pruned sweep: B=16 H=32 Dh=64 fp16, 8192 cached keys, 64 steps, 32 peaked keys/head, "
-                        "query fixed per head", "algorithmic_bytes_per_step": round(bytes_full), "results": res}
+    return {"workload": f"pruned sweep: B={B} H=32 Dh=64 fp16, 8192 cached keys, 64 steps, 32 peaked keys/head, "
+                        "query fixed per head", "launch": kind, "algorithmic_bytes_per_step": round(bytes_full),
+            "results": res}
+
+
+def run_pruned_sweeps():
+    for B, kind in ((16, "library"), (16, "workgroup"), (16, "two_pass"), (1, "library"), (1, "workgroup")):
+        print(json.dumps(run_pruned_sweep(B, kind)), flush=True)
+        import torch
+        torch.cuda.empty_cache()
 
 
 def run_suite(args):
@@ -335,7 +359,7 @@ def run_suite(args):
             del wl
             import torch
             torch.cuda.empty_cache()
-    print(json.dumps(run_pruned_sweep()), flush=True)
+    run_pruned_sweeps()
 
 
 def run_copy_calibration(mib=128, reps=40):
@@ -404,7 +428,7 @@ def main():
         run_suite(args)
         return
     if args.pruned_sweep:
-        print(json.dumps(run_pruned_sweep()))
+        run_pruned_sweeps()
         return
 
     plan_override = tuple(int(x) for x in args.plan.split(",")) if args.plan else None

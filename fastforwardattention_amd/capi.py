@@ -16,6 +16,7 @@ FFA_PRECISION_F16 = 16
 FFA_PRECISION_F32 = 32
 FFA_LAUNCH_WORKGROUP = 0
 FFA_LAUNCH_SPLIT = 1
+FFA_LAUNCH_TWO_PASS = 2
 FFA_COMBINE_FUSED = 0
 FFA_COMBINE_KERNEL = 1
 
@@ -25,6 +26,7 @@ STATUS_NAMES = {
     8: "FFA_ERR_PLAN", 9: "FFA_ERR_TOO_LONG", 10: "FFA_ERR_PROB_THRESH", 11: "FFA_ERR_LAUNCH",
     12: "FFA_ERR_NO_DEVICE",
 }
+globals().update({name: code for code, name in STATUS_NAMES.items()})   # FFA_OK, FFA_ERR_* as ints
 
 
 class LaunchPlan(C.Structure):

@@ -36,21 +36,36 @@ int run_decode(const DecodeArgs& a, const ffa_launch_plan* user_plan, void* work
     if (user_plan != nullptr) {
         plan = *user_plan;
     } else {
-        // Diagnostics exist only in the one-workgroup kernel.
-        st = plan_launch(a.precision, a.B, a.H, a.Dh, a.t, a.p, /*use_default=*/0,
-                         diag ? 256 : query_compute_units(), &plan);
-        if (st == FFA_OK && diag && plan.kind != FFA_LAUNCH_WORKGROUP)
-            st = plan_launch(a.precision, a.B, a.H, a.Dh, a.t, 1.f, 0, 256, &plan);
+        // Diagnostics do not exist in the exact split kernel: plan as for a pruned step.
+        const int cus = query_compute_units();
+        st = plan_launch(a.precision, a.B, a.H, a.Dh, a.t, a.p, /*use_default=*/0, cus, &plan);
+        if (st == FFA_OK && diag && plan.kind == FFA_LAUNCH_SPLIT)
+            st = plan_launch(a.precision, a.B, a.H, a.Dh, a.t, 1.f, 0, cus, &plan);
         if (st != FFA_OK) return st;
     }
     st = validate_plan(plan, a.precision, a.B * a.H, a.t, a.p);
     if (st != FFA_OK) return st;
-    if (diag && plan.kind != FFA_LAUNCH_WORKGROUP) return FFA_ERR_PLAN;
+    if (diag && plan.kind == FFA_LAUNCH_SPLIT) return FFA_ERR_PLAN;
 
-    WorkspaceView ws = {nullptr, nullptr, nullptr};
+    WorkspaceView ws = {nullptr, nullptr, nullptr, nullptr, 0};
     const int bh = a.B * a.H;
     const int split_heads = bh - plan.whole_heads;
-    if (plan.kind == FFA_LAUNCH_SPLIT && plan.n_splits > 1 && split_heads > 0) {
+    if (plan.kind == FFA_LAUNCH_TWO_PASS) {
+        // [counters][piece (max, sum)][partial outputs][scores]
+        if (workspace == nullptr ||
+            workspace_bytes < two_pass_workspace_bytes(bh, a.Dh, plan.n_splits, a.Lmax))
+            return FFA_ERR_WORKSPACE;
+        if (!aligned16(workspace)) return FFA_ERR_ALIGNMENT;
+        char* base = static_cast<char*>(workspace);
+        ws.cnt = reinterpret_cast<unsigned int*>(base);
+        base += workspace_counter_bytes(bh);
+        ws.ml = reinterpret_cast<float*>(base);
+        base += align_up((size_t)bh * plan.n_splits * 2 * sizeof(float), 256);
+        ws.acc = reinterpret_cast<float*>(base);
+        base += align_up((size_t)bh * plan.n_splits * a.Dh * sizeof(float), 256);
+        ws.scores = reinterpret_cast<float*>(base);
+        ws.score_stride = score_stride_for(a.Lmax);
+    } else if (plan.kind == FFA_LAUNCH_SPLIT && plan.n_splits > 1 && split_heads > 0) {
         if (workspace == nullptr ||
             workspace_bytes < workspace_bytes_for(bh, split_heads, a.Dh, plan.n_splits))
             return FFA_ERR_WORKSPACE;
@@ -118,7 +133,10 @@ int ffa_plan_launch(int precision, int batch_size, int head_num, int head_dim, i
 size_t ffa_workspace_bytes(int batch_size, int head_num, int head_dim, int max_seq_len) {
     if (batch_size <= 0 || head_num <= 0 || head_dim <= 0 || max_seq_len <= 0) return 0;
     const int bh = batch_size * head_num;
-    return workspace_bytes_for(bh, bh, head_dim, max_splits_for(bh, max_seq_len));
+    const int n_splits = max_splits_for(bh, max_seq_len);
+    const size_t exact = workspace_bytes_for(bh, bh, head_dim, n_splits);
+    const size_t two_pass = two_pass_workspace_bytes(bh, head_dim, n_splits, max_seq_len);
+    return exact > two_pass ? exact : two_pass;
 }
 
 int ffa_workspace_init(void* workspace, size_t workspace_bytes, void* stream) {

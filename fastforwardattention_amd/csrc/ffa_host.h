@@ -31,8 +31,10 @@ struct DecodeArgs {
 // Carved-up workspace for a given plan.
 struct WorkspaceView {
     unsigned int* cnt;  // [B*H] arrival counters, zero between launches
-    float* ml;          // [B*H, n_splits, 2]
-    float* acc;         // [B*H, n_splits, Dh]
+    float* ml;          // [split pairs, n_splits, 2]
+    float* acc;         // [split pairs, n_splits, Dh]
+    float* scores;      // two-pass path: [B*H, score_stride] raw scores
+    int score_stride;
 };
 
 inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
@@ -64,6 +66,15 @@ inline size_t workspace_bytes_for(int bh, int split_heads, int head_dim, int n_s
     if (n_splits <= 1 || split_heads <= 0) return workspace_counter_bytes(bh);
     return workspace_counter_bytes(bh) + align_up((size_t)split_heads * n_splits * 2 * sizeof(float), 256) +
            (size_t)split_heads * n_splits * head_dim * sizeof(float);
+}
+
+// Two-pass path: counters, piece (max, sum) [bh, n_splits, 2], partial outputs
+// [bh, n_splits, Dh], scores [bh, stride].
+inline int score_stride_for(int max_seq_len) { return (max_seq_len / kTileKeys + 1) * kTileKeys; }
+inline size_t two_pass_workspace_bytes(int bh, int head_dim, int n_splits, int max_seq_len) {
+    return workspace_counter_bytes(bh) + align_up((size_t)bh * n_splits * 2 * sizeof(float), 256) +
+           align_up((size_t)bh * n_splits * head_dim * sizeof(float), 256) +
+           align_up((size_t)bh * score_stride_for(max_seq_len) * sizeof(float), 256);
 }
 
 // planner (ffa_plan.cpp)

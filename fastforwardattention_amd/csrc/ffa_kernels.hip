@@ -13,7 +13,8 @@
 // computed in the K mapping (one key per lane) reach the V mapping (one row per LPR lanes)
 // through a 256-byte LDS stage per wave.
 //
-// Two decode kernels:
+// Decode kernels (the two-pass pair ffa_scores_kernel / ffa_pruned_pv_kernel is described
+// where it is defined):
 //   ffa_decode_split_kernel  p == 0.  Grid (b,h,split); every wave walks 64-key tiles with
 //     an online softmax, the waves of a workgroup merge (m, l, acc) in LDS, workgroups
 //     write partials and the last one to arrive (device-scope counter) merges them.
@@ -41,6 +42,8 @@ struct DecodeParams {
     float* ws_acc;         // [BH, n_splits, Dh]
     float* ws_ml;          // [BH, n_splits, 2]
     unsigned int* ws_cnt;  // [BH]
+    float* ws_scores;      // [BH, score_stride] raw q.k of the two-pass path
+    int score_stride;      // floats per (b,h) row of ws_scores, a multiple of 64
     unsigned int* kept_count;
     unsigned char* skip_mask;
     int B, H, Lmax, t;
@@ -648,6 +651,236 @@ __global__ void __launch_bounds__(NW * 64) ffa_decode_wg_kernel(const DecodePara
 }
 
 // ---------------------------------------------------------------------------------------
+// Two-pass sequence-split path (FFA_LAUNCH_TWO_PASS): any p, any length, n_splits pieces per
+// (b,h) pair.  Pass 1 streams K and leaves the raw scores (4 bytes per key) and each piece's
+// (max, sum of exp2) in the workspace; pass 2 folds those into the pair's global max and sum
+// -- which the pruning rule needs before it may touch a single V row -- then streams only
+// the V rows that survive.  Weights are normalised globally, hence the pieces' partial
+// outputs simply add up (merged by the last piece to arrive).
+template <typename T, int DH, int NW>
+__global__ void __launch_bounds__(NW * 64) ffa_scores_kernel(const DecodeParams P) {
+    using G = Geo<T, DH>;
+    constexpr int NCH = G::NCH;
+    __shared__ float s_m[NW], s_l[NW];
+    __shared__ uint4 s_q[G::Q_LDS ? NCH : 1];
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int bh = blockIdx.x / P.n_splits, split = blockIdx.x % P.n_splits;
+    const int b = bh / P.H;
+    int tlen, first;
+    step_bounds(P, b, tlen, first);
+
+    const size_t head_bytes = (size_t)P.Lmax * DH * sizeof(T);
+    char* kc_bh = reinterpret_cast<char*>(P.k_cache) + (size_t)bh * head_bytes;
+    char* vc_bh = reinterpret_cast<char*>(P.v_cache) + (size_t)bh * head_bytes;
+    const char* knew = reinterpret_cast<const char*>(P.k) + (size_t)bh * DH * sizeof(T);
+    const char* vnew = reinterpret_cast<const char*>(P.v) + (size_t)bh * DH * sizeof(T);
+    const uint4* qg = reinterpret_cast<const uint4*>(reinterpret_cast<const char*>(P.q) +
+                                                     (size_t)bh * DH * sizeof(T));
+    uint4 q_reg[G::QREG];
+    if constexpr (G::Q_LDS) {
+        if (tid < NCH) s_q[tid] = qg[tid];
+        __syncthreads();
+    } else {
+#pragma unroll
+        for (int c = 0; c < NCH; ++c) q_reg[c] = qg[c];
+    }
+
+    const int ntiles = tlen / kWave + 1;
+    const int tile_lo = max(split * P.tiles_per_split, first / kWave);
+    const int tile_hi = min(ntiles, (split + 1) * P.tiles_per_split);
+    const bool appends = split == min((ntiles - 1) / P.tiles_per_split, P.n_splits - 1) && wave == 0;
+    NewToken new_tok;
+    if (appends) new_tok = new_token_load<NCH>(knew, vnew, lane);
+    if (split == 0 && tid == 0 && P.kept_count) P.kept_count[bh] = 0u;  // pass 2 accumulates
+
+    // Each lane keeps a running (max, sum of exp2) over its own keys; lanes, then waves, are
+    // folded once at the end.
+    float* sc = P.ws_scores + (size_t)bh * P.score_stride;
+    float m_run = -INFINITY, l_run = 0.f;
+    for (int tile = tile_lo + wave; tile < tile_hi; tile += NW) {
+        const int key = tile * kWave + lane;
+        const float s = tile_qk<T, NCH, G::Q_LDS>(kc_bh, knew, key, tlen, P.Lmax, q_reg, s_q);
+        const bool valid = key <= tlen && key >= first;
+        sc[key] = valid ? s : -INFINITY;  // raw dot product; the whole 64-key tile is written
+        if (valid) {
+            const float m_new = fmaxf(m_run, s * P.scale_log2e);
+            l_run = l_run * __builtin_amdgcn_exp2f(m_run - m_new) +
+                    __builtin_amdgcn_exp2f(fmaf(s, P.scale_log2e, -m_new));
+            m_run = m_new;
+        }
+    }
+    if (appends) new_token_store<NCH>(new_tok, kc_bh, vc_bh, tlen, P.Lmax, lane);
+    const float m_w = wave_max(m_run);
+    const float l_w = wave_sum(m_run == -INFINITY ? 0.f : l_run * __builtin_amdgcn_exp2f(m_run - m_w));
+    if (lane == 0) {
+        s_m[wave] = m_w;
+        s_l[wave] = l_w;
+    }
+    __syncthreads();
+    if (tid == 0) {
+        float M = -INFINITY, L = 0.f;
+#pragma unroll
+        for (int w = 0; w < NW; ++w) M = fmaxf(M, s_m[w]);
+#pragma unroll
+        for (int w = 0; w < NW; ++w)
+            if (s_m[w] != -INFINITY) L += s_l[w] * __builtin_amdgcn_exp2f(s_m[w] - M);
+        float* ml = P.ws_ml + ((size_t)bh * P.n_splits + split) * 2;
+        ml[0] = M;
+        ml[1] = L;
+    }
+}
+
+template <typename T, int DH, int NW>
+__global__ void __launch_bounds__(NW * 64) ffa_pruned_pv_kernel(const DecodeParams P) {
+    using G = Geo<T, DH>;
+    constexpr int X = G::X, NCH = G::NCH, LPR = G::LPR, RPI = G::RPI;
+    constexpr int VG = NCH < 8 ? NCH : 8;
+    constexpr int NT = NW * 64;
+    __shared__ float s_p[NW][kWave];
+    __shared__ float s_acc[NW][DH];
+    __shared__ unsigned s_cnt[NW];
+    __shared__ int s_last;
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int bh = blockIdx.x / P.n_splits, split = blockIdx.x % P.n_splits;
+    const int b = bh / P.H;
+    int tlen, first;
+    step_bounds(P, b, tlen, first);
+
+    const size_t head_bytes = (size_t)P.Lmax * DH * sizeof(T);
+    const char* vc_bh = reinterpret_cast<const char*>(P.v_cache) + (size_t)bh * head_bytes;
+    const char* vnew = reinterpret_cast<const char*>(P.v) + (size_t)bh * DH * sizeof(T);
+    const float* sc = P.ws_scores + (size_t)bh * P.score_stride;
+
+    const int ntiles = tlen / kWave + 1;
+    const int tile_first = min(first / kWave, ntiles);  // tiles below are fully masked
+    const int tile_lo = max(split * P.tiles_per_split, tile_first);
+    const int tile_hi = min(ntiles, (split + 1) * P.tiles_per_split);
+    const bool pruned = P.p > 0.f;
+
+    // ---- the pair's max and sum from the pieces' (max, sum): every workgroup of the pair
+    // folds them in the same order, so all of them arrive at bit-identical M, S ----
+    const float* ml = P.ws_ml + (size_t)bh * P.n_splits * 2;
+    float M = -INFINITY;
+    for (int s = 0; s < P.n_splits; ++s) M = fmaxf(M, ml[2 * s]);
+    const bool all_masked = (M == -INFINITY);
+    if (all_masked) M = 0.f;
+    float S = 0.f;
+    for (int s = 0; s < P.n_splits; ++s) {
+        const float m_s = ml[2 * s];
+        if (m_s != -INFINITY) S += ml[2 * s + 1] * __builtin_amdgcn_exp2f(m_s - M);
+    }
+
+    // p == 0: exact softmax weights e_i / S.  p > 0: the reference's rule
+    // (attention.cu:1122-1126, :1184-1191), as in ffa_decode_wg_kernel.
+    const float inv = pruned ? 1.f / (S + 1.e-6f) : (S > 0.f ? 1.f / S : 0.f);
+    float thr_key = 0.f;
+    if (pruned) (void)round_prob(P.p * inv, T{}, &thr_key);
+
+    // ---- own tiles: weights (one key per lane) -> LDS stage -> surviving V rows ----
+    const int rg = lane / LPR, dch = lane % LPR;
+    float acc[X];
+#pragma unroll
+    for (int e = 0; e < X; ++e) acc[e] = 0.f;
+    unsigned kept = 0;
+    for (int tile = tile_lo + wave; tile < tile_hi; tile += NW) {
+        const int key = tile * kWave + lane;
+        const float sr = sc[key];
+        const float e = (sr == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(fmaf(sr, P.scale_log2e, -M));
+        const bool in_range = key >= first && key <= tlen;
+        float w;
+        bool drop;
+        if (pruned) {
+            float key_i;
+            w = round_prob(e * inv, T{}, &key_i);
+            drop = !in_range || (key < tlen && key_i <= thr_key);
+        } else {
+            w = e * inv;
+            drop = !in_range;
+        }
+        if (key < tlen) {
+            kept += drop ? 0u : 1u;
+            if (P.skip_mask) P.skip_mask[(size_t)bh * P.Lmax + key] = drop ? 1 : 0;
+        }
+        __builtin_amdgcn_wave_barrier();
+        s_p[wave][stage_slot<NCH, RPI>(lane)] = drop ? -1.f : w;
+        __builtin_amdgcn_wave_barrier();
+        const float* pst = &s_p[wave][rg * NCH];
+#pragma unroll 1
+        for (int g = 0; g < NCH / VG; ++g) {
+            uint4 vv[VG];
+            float pj[VG];
+#pragma unroll
+            for (int j = 0; j < VG; ++j) {
+                const int row = tile * kWave + (g * VG + j) * RPI + rg;
+                pj[j] = pst[g * VG + j];
+                vv[j] = make_uint4(0, 0, 0, 0);
+                if (pj[j] >= 0.f) {
+                    const char* vp = row < tlen ? vc_bh + ((size_t)row * NCH + dch) * 16 : vnew + dch * 16;
+                    vv[j] = ld16(vp);
+                } else {
+                    pj[j] = 0.f;
+                }
+            }
+#pragma unroll
+            for (int j = 0; j < VG; ++j) fma_chunk(acc, pj[j], vv[j], T{});
+        }
+        __builtin_amdgcn_wave_barrier();
+    }
+    if (P.skip_mask && split == 0)  // keys of fully masked leading tiles are dropped too
+        for (int i = tid; i < min(tile_first * kWave, tlen); i += NT) P.skip_mask[(size_t)bh * P.Lmax + i] = 1;
+
+    // ---- merge: lanes of a wave, waves of the workgroup, pieces of the pair ----
+#pragma unroll
+    for (int off = LPR; off < kWave; off <<= 1) {
+#pragma unroll
+        for (int e = 0; e < X; ++e) acc[e] += __shfl_xor(acc[e], off);
+    }
+    if (lane < LPR) {
+#pragma unroll
+        for (int e = 0; e < X; ++e) s_acc[wave][lane * X + e] = acc[e];
+    }
+    kept = wave_sum_u32(kept);
+    if (lane == 0) s_cnt[wave] = kept;
+    __syncthreads();
+    if (P.kept_count && tid == 0) {
+        unsigned tot = 0;
+#pragma unroll
+        for (int w = 0; w < NW; ++w) tot += s_cnt[w];
+        if (tot) atomicAdd(&P.kept_count[bh], tot);
+    }
+
+    T* out = reinterpret_cast<T*>(P.out) + (size_t)bh * DH;
+    float* wa = P.ws_acc + ((size_t)bh * P.n_splits + split) * DH;
+    for (int d = tid; d < DH; d += NT) {
+        float o = 0.f;
+#pragma unroll
+        for (int w = 0; w < NW; ++w) o += s_acc[w][d];
+        if (P.n_splits == 1) store_out(out, d, all_masked ? 0.f : o);
+        else publish(&wa[d], o);
+    }
+    if (P.n_splits == 1) return;
+
+    // Same publication protocol as ffa_decode_split_kernel (device-scope relaxed atomics,
+    // ordered by the workgroup barrier and the arrival counter; no fences).
+    __syncthreads();
+    if (tid == 0) {
+        const unsigned prev =
+            __hip_atomic_fetch_add(&P.ws_cnt[bh], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        s_last = (prev == (unsigned)(P.n_splits - 1));
+    }
+    __syncthreads();
+    if (!s_last) return;
+    for (int d = tid; d < DH; d += NT) {
+        float o = 0.f;
+        for (int s = 0; s < P.n_splits; ++s) o += acquire(&P.ws_acc[((size_t)bh * P.n_splits + s) * DH + d]);
+        store_out(out, d, all_masked ? 0.f : o);
+    }
+    if (tid == 0) __hip_atomic_store(&P.ws_cnt[bh], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// ---------------------------------------------------------------------------------------
 // Cache construction (attention.cu:1556-1609).  One workgroup moves a tile of TK keys of
 // one (b,h): coalesced row reads [64 keys x Dh] -> LDS -> coalesced 1 KiB chunk-row writes
 // for K; V is a straight strided copy.
@@ -701,6 +934,14 @@ static int launch_split(const DecodeParams& P, hipStream_t st) {
 }
 
 template <typename T, int DH, int NW>
+static int launch_two_pass(const DecodeParams& P, hipStream_t st) {
+    const dim3 grid((unsigned)(P.bh_total * P.n_splits));
+    hipLaunchKernelGGL((ffa_scores_kernel<T, DH, NW>), grid, dim3(NW * 64), 0, st, P);
+    hipLaunchKernelGGL((ffa_pruned_pv_kernel<T, DH, NW>), grid, dim3(NW * 64), 0, st, P);
+    return check_launch();
+}
+
+template <typename T, int DH, int NW>
 static int launch_wg(const DecodeParams& P, size_t lds_bytes, hipStream_t st) {
     auto kern = ffa_decode_wg_kernel<T, DH, NW>;
     if (lds_bytes > 48 * 1024) {
@@ -728,6 +969,15 @@ static int dispatch_waves(const DecodeParams& P, const ffa_launch_plan& plan, hi
             case 2: return launch_split<T, DH, 2>(P, st);
             case 4: return launch_split<T, DH, 4>(P, st);
             case 8: return launch_split<T, DH, 8>(P, st);
+            default: return FFA_ERR_PLAN;
+        }
+    }
+    if (plan.kind == FFA_LAUNCH_TWO_PASS) {
+        switch (plan.waves_per_wg) {
+            case 1: return launch_two_pass<T, DH, 1>(P, st);
+            case 2: return launch_two_pass<T, DH, 2>(P, st);
+            case 4: return launch_two_pass<T, DH, 4>(P, st);
+            case 8: return launch_two_pass<T, DH, 8>(P, st);
             default: return FFA_ERR_PLAN;
         }
     }
@@ -764,6 +1014,7 @@ int launch_decode(const DecodeArgs& a, const ffa_launch_plan& plan, const Worksp
     P.k_cache = a.k_cache; P.v_cache = a.v_cache; P.out = a.out;
     P.seq_lengths = a.seq_lengths;
     P.ws_acc = ws.acc; P.ws_ml = ws.ml; P.ws_cnt = ws.cnt;
+    P.ws_scores = ws.scores; P.score_stride = ws.score_stride;
     P.kept_count = a.kept_count; P.skip_mask = a.skip_mask;
     P.B = a.B; P.H = a.H; P.Lmax = a.Lmax; P.t = a.t;
     P.scale_log2e = a.scale * kLog2e;

@@ -57,17 +57,34 @@ int plan_launch(int precision, int B, int H, int Dh, int t, float p, int use_def
     if (use_default) {
         // One workgroup per (batch, head); workgroup size by sequence length like the
         // FasterTransformer table (kernel_launch_utils.h:147-154: 64 / 128 / 256 threads).
-        if (!fits_wg) return FFA_ERR_TOO_LONG;
+        // Sequences whose scores outgrow LDS keep them in the workspace instead.
         const int waves = t < 32 ? 1 : (t < 2048 ? 2 : 4);
-        fill(plan, FFA_LAUNCH_WORKGROUP, wg_waves_for(ntiles, waves), 1, ntiles);
+        fill(plan, fits_wg ? FFA_LAUNCH_WORKGROUP : FFA_LAUNCH_TWO_PASS, wg_waves_for(ntiles, waves), 1,
+             ntiles);
         return FFA_OK;
     }
 
     if (p > 0.f) {
-        // Pruning needs the global max and sum before V: one workgroup per (b,h), as many
-        // waves as there are tiles to keep in flight (up to 16).
-        if (!fits_wg) return FFA_ERR_TOO_LONG;
-        fill(plan, FFA_LAUNCH_WORKGROUP, wg_waves_for(ntiles, ceil_div(ntiles, 4)), 1, ntiles);
+        // Pruning needs the global max and sum before it may touch V.  With at least half a
+        // pair per CU and scores that fit LDS: one workgroup per (b,h), as many waves as
+        // there are tiles to keep in flight (up to 16).  Otherwise the two-pass pair of
+        // kernels, cut into floor(CUs/pairs) pieces per pair like the exact path.
+        if (fits_wg && 2 * bh >= cus) {
+            fill(plan, FFA_LAUNCH_WORKGROUP, wg_waves_for(ntiles, ceil_div(ntiles, 4)), 1, ntiles);
+            return FFA_OK;
+        }
+        const int waves = wg_waves_for(ntiles, 4);
+        int n_splits = cus / bh;
+        if (n_splits > ceil_div(ntiles, waves)) n_splits = ceil_div(ntiles, waves);
+        const int cap = max_splits_for(bh, t + 1);
+        if (n_splits > cap) n_splits = cap;
+        if (n_splits < 1) n_splits = 1;
+        const int tps = ceil_div(ntiles, n_splits);
+        n_splits = ceil_div(ntiles, tps);
+        if (n_splits == 1 && fits_wg)  // nothing to cut: the single kernel does the same work
+            fill(plan, FFA_LAUNCH_WORKGROUP, wg_waves_for(ntiles, ceil_div(ntiles, 4)), 1, ntiles);
+        else
+            fill(plan, FFA_LAUNCH_TWO_PASS, waves, n_splits, tps);
         return FFA_OK;
     }
 
@@ -122,6 +139,11 @@ int validate_plan(const ffa_launch_plan& plan, int precision, int bh, int t, flo
                 return FFA_ERR_PLAN;
             if ((long long)(bh - plan.whole_heads) * plan.n_splits > 4 * kMaxSplitWorkgroups)
                 return FFA_ERR_PLAN;
+            return FFA_OK;
+        case FFA_LAUNCH_TWO_PASS:
+            if (w > 8 || plan.whole_heads != 0 || plan.combine != FFA_COMBINE_FUSED) return FFA_ERR_PLAN;
+            if ((long long)plan.n_splits * plan.tiles_per_split < ntiles) return FFA_ERR_PLAN;
+            if ((long long)bh * plan.n_splits > 4 * kMaxSplitWorkgroups) return FFA_ERR_PLAN;
             return FFA_OK;
         default:
             return FFA_ERR_PLAN;

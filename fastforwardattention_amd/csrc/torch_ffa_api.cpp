@@ -209,7 +209,7 @@ private:
 
         ffa_launch_plan plan;
         const bool diag = kept != nullptr || mask != nullptr;
-        // Diagnostics exist in the one-workgroup launch only.
+        // The default launch keeps diagnostics at any length; the exact split kernel has none.
         check_status(ffa_plan_launch(precision, d.B, d.H, d.Dh, t, prob_thresh,
                                      (ft_kernel_launch || diag) ? 1 : 0, 0, &plan),
                      "launch planning");

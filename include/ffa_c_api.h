@@ -42,7 +42,7 @@ typedef enum ffa_status {
     FFA_ERR_ALIGNMENT = 6,      /* a pointer is not 16-byte aligned                          */
     FFA_ERR_WORKSPACE = 7,      /* workspace NULL/too small for the chosen plan              */
     FFA_ERR_PLAN = 8,           /* malformed launch plan                                     */
-    FFA_ERR_TOO_LONG = 9,       /* t+1 scores do not fit the LDS of a one-workgroup launch   */
+    FFA_ERR_TOO_LONG = 9,       /* t+1 scores do not fit the LDS of an FFA_LAUNCH_WORKGROUP plan */
     FFA_ERR_PROB_THRESH = 10,   /* p is negative or NaN                                      */
     FFA_ERR_LAUNCH = 11,        /* the HIP runtime refused the launch                        */
     FFA_ERR_NO_DEVICE = 12      /* no usable gfx950 device / HIP runtime error               */
@@ -59,6 +59,9 @@ typedef enum ffa_status {
 #define FFA_LAUNCH_SPLIT 1      /* online-softmax kernel, p == 0 only: whole_heads pairs    */
                                 /* with one workgroup each, the others split over n_splits  */
                                 /* workgroups whose partials the last arriver combines      */
+#define FFA_LAUNCH_TWO_PASS 2   /* any p >= 0, any length: a scores kernel (K stream, raw   */
+                                /* scores to the workspace) then a weights x V kernel that  */
+                                /* reads only surviving rows; n_splits pieces per pair      */
 
 /* How the partial (max, sum, acc[Dh]) results of a split launch are merged. */
 #define FFA_COMBINE_FUSED 0     /* by the last workgroup of each (batch, head) to arrive     */
@@ -98,7 +101,7 @@ int ffa_plan_launch(int precision, int batch_size, int head_num, int head_dim,
                     int compute_units, ffa_launch_plan* plan);
 
 /* Bytes of device workspace sufficient for ANY plan this library produces for the
- * given problem (split partials + arrival counters). */
+ * given problem (arrival counters, split partials, two-pass scores). */
 size_t ffa_workspace_bytes(int batch_size, int head_num, int head_dim, int max_seq_len);
 
 /* Zero the arrival counters of a fresh workspace (once, before first use). */
@@ -149,8 +152,8 @@ int ffa_attention_f32(int batch_size, int head_num, int head_dim, int max_seq_le
  *   kept_count  device uint32[B*H] or NULL: number of cached keys i < t whose V row was
  *               read (overwritten, not accumulated);
  *   skip_mask   device uint8[B*H*Lmax] or NULL: 1 where key i < t was dropped.
- * Diagnostics need the one-workgroup launch: a NULL plan is planned that way, an
- * FFA_LAUNCH_SPLIT plan is rejected with FFA_ERR_PLAN.  With prob_thresh == 0 only
+ * The exact split kernel keeps no diagnostics: a NULL plan is planned as for a pruned
+ * step, an FFA_LAUNCH_SPLIT plan is rejected with FFA_ERR_PLAN.  With prob_thresh == 0 only
  * masked (left-padding) keys count as dropped and kept_count[b,h] = t - first_key.
  */
 int ffa_attention_diag(int precision, int batch_size, int head_num, int head_dim,

@@ -40,6 +40,11 @@ def _plans(prec, B, H, Dh, t):
             plans.append((f"split_w{waves}_tps{tps}", capi.make_plan(capi.FFA_LAUNCH_SPLIT, waves, ns, tps)))
             plans.append((f"split_w{waves}_tps{tps}_mergekernel",
                           capi.make_plan(capi.FFA_LAUNCH_SPLIT, waves, ns, tps, capi.FFA_COMBINE_KERNEL)))
+    # two-pass launches (scores kernel, then weights x V): same answer at p == 0
+    for waves, tps in [(1, 1), (4, 3), (8, 2), (2, ntiles)]:
+        ns = -(-ntiles // tps)
+        if ns <= 128:
+            plans.append((f"twopass_w{waves}_tps{tps}", capi.make_plan(capi.FFA_LAUNCH_TWO_PASS, waves, ns, tps)))
     # hybrid launches: some (batch, head) pairs whole, the rest split
     bh = B * H
     for whole in sorted({1, bh // 2, bh - 1, bh}):
@@ -242,9 +247,13 @@ def test_pruned_step_matches_rule(prec, Dh, L, p):
     scale = 1.0 / np.sqrt(Dh)   # peaked keys score 4*|q|*scale ~ 4 against N(0,1) for the rest
     want, skip, P, thr = O.pruned_decode_step(q, k, v, O.pack_k_cache(K, Lmax), O.pack_v_cache(V, Lmax),
                                               scale, L, p)
-    for waves in (1, 4, 16):
-        _say("pruned", prec, Dh, L, p, waves)
-        plan = capi.make_plan(capi.FFA_LAUNCH_WORKGROUP, waves, 1, L // 64 + 1)
+    ntiles = L // 64 + 1
+    plans = [capi.make_plan(capi.FFA_LAUNCH_WORKGROUP, waves, 1, ntiles) for waves in (1, 4, 16)]
+    plans += [capi.make_plan(capi.FFA_LAUNCH_TWO_PASS, waves, -(-ntiles // tps), tps)
+              for waves, tps in ((1, 1), (4, 2), (8, 5), (4, ntiles))]
+    plans.append(None)   # planned by the library: few pairs -> two-pass
+    for plan in plans:
+        _say("pruned", prec, Dh, L, p, plan)
         got, kept, gmask = CApiSession(K, V, Lmax).step(q, k, v, scale, L, p=p, plan=plan, diag=True)
         near = _near_threshold(prec, P, thr)
         diff = gmask != skip
@@ -270,6 +279,39 @@ def test_pruned_tiny_threshold_equals_exact(prec):
     exact = CApiSession(K, V, L + 1).step(q, k, v, 0.125, L, p=0.0, plan=plan)
     tiny = CApiSession(K, V, L + 1).step(q, k, v, 0.125, L, p=1e-30, plan=plan)
     assert np.abs(exact - tiny).max() <= (2e-3 if prec == 16 else 2e-6)
+
+
+@pytest.mark.parametrize("prec", [16, 32])
+def test_sequences_beyond_lds(prec):
+    """45001 keys: the scores no longer fit LDS, so pruned and default launches go through the
+    two-pass kernels; exact against the closed form, pruned against the rule."""
+    B, H, Dh, L = 1, 2, 64, 45000
+    K, V, q, k, v = _peaked(prec, 13, B, H, L, Dh)
+    Lmax, scale = L + 8, 0.125
+    kc0, vc0 = O.pack_k_cache(K, Lmax), O.pack_v_cache(V, Lmax)
+    want = O.decode_step(q, k, v, kc0, vc0, scale, L, acc=np.float64)
+    wg = capi.make_plan(capi.FFA_LAUNCH_WORKGROUP, 16, 1, L // 64 + 1)
+    CApiSession(K[:, :, :8], V[:, :, :8], Lmax).step(q, k, v, scale, L, plan=wg, expect=capi.FFA_ERR_TOO_LONG)
+    for name, plan in (("default", capi.plan_launch(prec, B, H, Dh, L, 0.0, True)), ("tuned", None)):
+        _say("beyond_lds exact", prec, name)
+        sess = CApiSession(K, V, Lmax)
+        got = sess.step(q, k, v, scale, L, plan=plan)
+        assert float(np.abs(got - want).max()) <= _tol(prec, V, v), name
+        gk, gv = sess.caches()
+        np.testing.assert_array_equal(gk[..., :L + 1, :], kc0[..., :L + 1, :])
+        np.testing.assert_array_equal(gv[:, :, :L + 1], vc0[:, :, :L + 1])
+    p = 0.05     # the rule compares exp(s_i - max) with p: peaks sit ~4.5 above the N(0,1) bulk
+    want_p, skip, P, thr = O.pruned_decode_step(q, k, v, kc0, vc0, scale, L, p)
+    for name, plan in (("default", capi.plan_launch(prec, B, H, Dh, L, p, True)), ("tuned", None)):
+        _say("beyond_lds pruned", prec, name)
+        got, kept, gmask = CApiSession(K, V, Lmax).step(q, k, v, scale, L, p=p, plan=plan, diag=True)
+        diff = gmask != skip
+        assert not (diff & ~_near_threshold(prec, P, thr)).any()
+        np.testing.assert_array_equal(kept, (L - gmask[:, :, :L].sum(axis=-1)))
+        Vall = np.concatenate([V, v[:, :, None]], axis=2).astype(np.float32)
+        w = np.where(gmask[:, :, :L + 1], 0, P[:, :, :L + 1])
+        assert float(np.abs(got - np.einsum("bhn,bhnd->bhd", w, Vall)).max()) <= (1e-3 if prec == 16 else 1e-5)
+    assert skip[:, :, :L].mean() > 0.5
 
 
 # ------------------------------------------------------------------ full-size properties

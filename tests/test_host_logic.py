@@ -117,6 +117,14 @@ def test_workspace_bytes_covers_every_plan(lib):
                     if plan.n_splits > 1 and sh > 0:
                         need += -(-sh * plan.n_splits * 8 // 256) * 256 + sh * plan.n_splits * Dh * 4
                     assert need <= total, (B, H, Dh, Lmax, t, plan)
+                    for p_, dflt in ((1e-3, False), (0.0, True)):
+                        plan = capi.plan_launch(prec, B, H, Dh, t, p_, dflt, cus)
+                        if plan.kind != capi.FFA_LAUNCH_TWO_PASS:
+                            continue
+                        up = lambda v: -(-v // 256) * 256
+                        need = (up(bh * 4) + up(bh * plan.n_splits * 8) + up(bh * plan.n_splits * Dh * 4) +
+                                up(bh * (Lmax // 64 + 1) * 64 * 4))
+                        assert need <= total, (B, H, Dh, Lmax, t, plan)
     assert lib.ffa_workspace_bytes(0, 1, 64, 8) == 0
 
 
@@ -132,8 +140,19 @@ def test_planner_consistency(prec, Dh):
                     assert plan.threads_per_key == 1 and plan.keys_per_wave == 64
                     assert plan.waves_per_wg in (1, 2, 4, 8, 16)
                     assert plan.n_splits * plan.tiles_per_split >= ntiles      # every key covered
-                    if use_default or p > 0:
-                        assert plan.kind == capi.FFA_LAUNCH_WORKGROUP and plan.n_splits == 1
+                    fits_lds = ntiles * 64 * 4 <= 156 * 1024
+                    if use_default:
+                        assert plan.n_splits == 1
+                        assert plan.kind == (capi.FFA_LAUNCH_WORKGROUP if fits_lds else capi.FFA_LAUNCH_TWO_PASS)
+                    elif p > 0:
+                        if plan.kind == capi.FFA_LAUNCH_WORKGROUP:
+                            assert plan.n_splits == 1 and fits_lds
+                        else:
+                            assert plan.kind == capi.FFA_LAUNCH_TWO_PASS
+                            assert plan.n_splits > 1 or not fits_lds
+                            assert (plan.n_splits - 1) * plan.tiles_per_split < ntiles  # no empty piece
+                            assert B * H * plan.n_splits <= max(256, B * H)              # about one per CU
+                            assert plan.waves_per_wg <= 8 and plan.whole_heads == 0
                     else:
                         assert plan.kind == capi.FFA_LAUNCH_SPLIT
                         assert (plan.n_splits - 1) * plan.tiles_per_split < ntiles  # no empty split
@@ -161,8 +180,21 @@ def test_planner_rejects_bad_input(lib):
     assert f(16, 1, 1, 64, -1, 0.0, 0, 256, C.byref(plan)) == 5
     assert f(16, 1, 1, 64, 10, -1.0, 0, 256, C.byref(plan)) == 10
     assert f(16, 1, 1, 64, 10, 0.0, 0, 256, None) == 1
-    assert f(16, 1, 1, 64, 50000, 0.5, 0, 256, C.byref(plan)) == 9   # pruned: scores must fit LDS
-    assert f(16, 1, 1, 64, 50000, 0.0, 1, 256, C.byref(plan)) == 9
+
+
+def test_planner_long_sequences_leave_lds():
+    # 50001 scores do not fit LDS: pruned and default launches keep them in the workspace
+    for p, default in ((0.5, False), (0.0, True), (0.5, True)):
+        plan = capi.plan_launch(16, 1, 1, 64, 50000, p, default, 256)
+        assert plan.kind == capi.FFA_LAUNCH_TWO_PASS
+        assert plan.n_splits * plan.tiles_per_split >= 50000 // 64 + 1
+    assert capi.plan_launch(16, 1, 1, 64, 50000, 0.0, True, 256).n_splits == 1
+    assert capi.plan_launch(16, 1, 1, 64, 50000, 0.5, False, 256).n_splits > 64
+    # few pairs, pruning on: cut along the sequence
+    plan = capi.plan_launch(16, 1, 32, 64, 8191, 1e-3, False, 256)
+    assert plan.kind == capi.FFA_LAUNCH_TWO_PASS and plan.n_splits == 8
+    # many pairs, scores fit: one workgroup per pair
+    assert capi.plan_launch(16, 16, 32, 64, 8191, 1e-3, False, 256).kind == capi.FFA_LAUNCH_WORKGROUP
 
 
 def test_extension_imports_and_refuses_cpu_tensors():
