@@ -759,18 +759,27 @@ __global__ void __launch_bounds__(NW * 64) ffa_pruned_pv_kernel(const DecodePara
     const int tile_hi = min(ntiles, (split + 1) * P.tiles_per_split);
     const bool pruned = P.p > 0.f;
 
-    // ---- the pair's max and sum from the pieces' (max, sum): every workgroup of the pair
-    // folds them in the same order, so all of them arrive at bit-identical M, S ----
+    // ---- the pair's max and sum from the pieces' (max, sum).  One piece per lane (two when
+    // n_splits > 64), all loads in flight at once; every wave of every workgroup of the pair
+    // folds them through the same reduction tree, so all arrive at bit-identical M, S ----
+    static_assert(kMaxSplits <= 2 * kWave, "two pieces per lane at most");
+    // The first tile's scores travel together with the pieces' (max, sum).
+    float sr_next = (tile_lo + wave < tile_hi) ? sc[(tile_lo + wave) * kWave + lane] : -INFINITY;
     const float* ml = P.ws_ml + (size_t)bh * P.n_splits * 2;
-    float M = -INFINITY;
-    for (int s = 0; s < P.n_splits; ++s) M = fmaxf(M, ml[2 * s]);
+    float m_a = -INFINITY, l_a = 0.f, m_b = -INFINITY, l_b = 0.f;
+    if (lane < P.n_splits) {
+        m_a = ml[2 * lane];
+        l_a = ml[2 * lane + 1];
+    }
+    if (lane + kWave < P.n_splits) {
+        m_b = ml[2 * (lane + kWave)];
+        l_b = ml[2 * (lane + kWave) + 1];
+    }
+    float M = wave_max(fmaxf(m_a, m_b));
     const bool all_masked = (M == -INFINITY);
     if (all_masked) M = 0.f;
-    float S = 0.f;
-    for (int s = 0; s < P.n_splits; ++s) {
-        const float m_s = ml[2 * s];
-        if (m_s != -INFINITY) S += ml[2 * s + 1] * __builtin_amdgcn_exp2f(m_s - M);
-    }
+    const float S = wave_sum((m_a == -INFINITY ? 0.f : l_a * __builtin_amdgcn_exp2f(m_a - M)) +
+                             (m_b == -INFINITY ? 0.f : l_b * __builtin_amdgcn_exp2f(m_b - M)));
 
     // p == 0: exact softmax weights e_i / S.  p > 0: the reference's rule
     // (attention.cu:1122-1126, :1184-1191), as in ffa_decode_wg_kernel.
@@ -786,7 +795,8 @@ __global__ void __launch_bounds__(NW * 64) ffa_pruned_pv_kernel(const DecodePara
     unsigned kept = 0;
     for (int tile = tile_lo + wave; tile < tile_hi; tile += NW) {
         const int key = tile * kWave + lane;
-        const float sr = sc[key];
+        const float sr = sr_next;
+        sr_next = (tile + NW < tile_hi) ? sc[key + NW * kWave] : -INFINITY;  // one tile ahead
         const float e = (sr == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(fmaf(sr, P.scale_log2e, -M));
         const bool in_range = key >= first && key <= tlen;
         float w;
@@ -872,9 +882,19 @@ __global__ void __launch_bounds__(NW * 64) ffa_pruned_pv_kernel(const DecodePara
     }
     __syncthreads();
     if (!s_last) return;
+    // All loads of a batch of pieces are issued before any is consumed.
+    constexpr int MB = 8;
     for (int d = tid; d < DH; d += NT) {
         float o = 0.f;
-        for (int s = 0; s < P.n_splits; ++s) o += acquire(&P.ws_acc[((size_t)bh * P.n_splits + s) * DH + d]);
+        for (int s0 = 0; s0 < P.n_splits; s0 += MB) {
+            float as[MB];
+#pragma unroll
+            for (int j = 0; j < MB; ++j)
+                as[j] = acquire(&P.ws_acc[((size_t)bh * P.n_splits + min(s0 + j, P.n_splits - 1)) * DH + d]);
+#pragma unroll
+            for (int j = 0; j < MB; ++j)
+                if (s0 + j < P.n_splits) o += as[j];
+        }
         store_out(out, d, all_masked ? 0.f : o);
     }
     if (tid == 0) __hip_atomic_store(&P.ws_cnt[bh], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);

@@ -68,19 +68,22 @@ int plan_launch(int precision, int B, int H, int Dh, int t, float p, int use_def
         // Pruning needs the global max and sum before it may touch V.  With at least half a
         // pair per CU and scores that fit LDS: one workgroup per (b,h), as many waves as
         // there are tiles to keep in flight (up to 16).  Otherwise the two-pass pair of
-        // kernels, cut into floor(CUs/pairs) pieces per pair like the exact path.
+        // kernels, cut along the sequence.
         if (fits_wg && 2 * bh >= cus) {
             fill(plan, FFA_LAUNCH_WORKGROUP, wg_waves_for(ntiles, ceil_div(ntiles, 4)), 1, ntiles);
             return FFA_OK;
         }
-        const int waves = wg_waves_for(ntiles, 4);
-        int n_splits = cus / bh;
-        if (n_splits > ceil_div(ntiles, waves)) n_splits = ceil_div(ntiles, waves);
+        // Measured on MI355X (8192 keys, 32 and 128 pairs): both kernels of the pair carry
+        // only half of a tile's loads each, so they want twice the workgroups of the exact
+        // path -- about two 8-wave workgroups per CU -- as long as every wave keeps a tile.
+        int n_splits = 2 * cus / bh;
+        if (n_splits > ntiles) n_splits = ntiles;
         const int cap = max_splits_for(bh, t + 1);
         if (n_splits > cap) n_splits = cap;
         if (n_splits < 1) n_splits = 1;
         const int tps = ceil_div(ntiles, n_splits);
         n_splits = ceil_div(ntiles, tps);
+        const int waves = wg_waves_for(tps, 8);
         if (n_splits == 1 && fits_wg)  // nothing to cut: the single kernel does the same work
             fill(plan, FFA_LAUNCH_WORKGROUP, wg_waves_for(ntiles, ceil_div(ntiles, 4)), 1, ntiles);
         else

@@ -108,7 +108,7 @@ def test_workspace_bytes_covers_every_plan(lib):
         total = lib.ffa_workspace_bytes(B, H, Dh, Lmax)
         assert total > 0
         for prec in (16, 32):
-            for t in sorted({0, 1, 63, 64, Lmax // 2, Lmax - 1}):
+            for t in sorted(t for t in {0, 1, 63, 64, Lmax // 2, Lmax - 1} if t < Lmax):
                 for cus in (64, 256, 304):
                     plan = capi.plan_launch(prec, B, H, Dh, t, 0.0, False, cus)
                     bh = B * H
@@ -151,7 +151,7 @@ def test_planner_consistency(prec, Dh):
                             assert plan.kind == capi.FFA_LAUNCH_TWO_PASS
                             assert plan.n_splits > 1 or not fits_lds
                             assert (plan.n_splits - 1) * plan.tiles_per_split < ntiles  # no empty piece
-                            assert B * H * plan.n_splits <= max(256, B * H)              # about one per CU
+                            assert B * H * plan.n_splits <= max(512, B * H)              # about two per CU
                             assert plan.waves_per_wg <= 8 and plan.whole_heads == 0
                     else:
                         assert plan.kind == capi.FFA_LAUNCH_SPLIT
@@ -192,7 +192,7 @@ def test_planner_long_sequences_leave_lds():
     assert capi.plan_launch(16, 1, 1, 64, 50000, 0.5, False, 256).n_splits > 64
     # few pairs, pruning on: cut along the sequence
     plan = capi.plan_launch(16, 1, 32, 64, 8191, 1e-3, False, 256)
-    assert plan.kind == capi.FFA_LAUNCH_TWO_PASS and plan.n_splits == 8
+    assert plan.kind == capi.FFA_LAUNCH_TWO_PASS and plan.n_splits == 16 and plan.waves_per_wg == 8
     # many pairs, scores fit: one workgroup per pair
     assert capi.plan_launch(16, 16, 32, 64, 8191, 1e-3, False, 256).kind == capi.FFA_LAUNCH_WORKGROUP
 
