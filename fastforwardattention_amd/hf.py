@@ -1,0 +1,242 @@
+"""Hugging Face decoder hook: routes the one-token decode steps of OPT- and GPT-J-style
+attention layers through `FastForwardAttn`.
+
+Stands where the reference patches transformers' model files in place (modeling_opt.py:196-226,
+modeling_gptj.py:252-281): the prompt pass runs ordinary attention and builds one
+`FastForwardAttn` per layer from the prompt's keys and values; every later call with a single
+query token goes to `attention(q, k, v, k_cache, v_cache, scale, t, seq_lens, p)` with
+`seq_lens` = index of the first real key of each left-padded sample (modeling_opt.py:222,
+modeling_gptj.py:274) and `t` = number of keys cached so far, carried per layer.
+
+Written against the installed transformers (5.x) instead of a patched copy of its files:
+
+* `FFACache` is a `transformers.Cache` whose layers own the engines.  Its `update` hands the
+  new token's key/value through (tagged with the layer that owns them) instead of returning
+  the concatenated history.
+* models that dispatch through transformers' attention-function registry (OPT) select the
+  registered function `"ffa"`; GPT-J, which calls its own `_attn`, gets that method wrapped.
+
+    from fastforwardattention_amd import hf
+    hf.enable(model)
+    out = model.generate(ids, attention_mask=mask, max_new_tokens=n,
+                         past_key_values=hf.FFACache(max_new_tokens=n))
+
+The reference's environment switches are honoured by `FFACache.from_env()`:
+`max_tokens`, `use_ffa_default_kl`, `prob_thresh` (summarize.py:77-96)."""
+from __future__ import annotations
+
+import functools
+import os
+import types
+
+import torch
+from transformers.cache_utils import Cache, CacheLayerMixin
+from transformers.masking_utils import AttentionMaskInterface, eager_mask
+from transformers.modeling_utils import AttentionInterface
+
+ATTN_NAME = "ffa"
+_TAG = "_ffa_layer"
+
+
+def _default_engine():
+    from . import FastForwardAttn  # raises ImportError when the HIP extension is not built
+    return FastForwardAttn
+
+
+class FFALayer(CacheLayerMixin):
+    """One decoder layer's cache: a `FastForwardAttn` built at the prompt pass, the number of
+    keys it holds, and the left-padding offsets of the batch."""
+
+    is_sliding = False
+    is_compileable = False
+
+    def __init__(self, max_new_tokens: int, prob_thresh: float = 0.0,
+                 use_default_kernel_launch: bool = False, engine=None):
+        super().__init__()
+        if max_new_tokens < 1:
+            raise ValueError("max_new_tokens must be >= 1")
+        self.max_new_tokens = int(max_new_tokens)
+        self.prob_thresh = float(prob_thresh)
+        self.use_default_kernel_launch = bool(use_default_kernel_launch)
+        self._engine_cls = engine
+        self.engine = None
+        self.t = 0                  # keys cached so far = slot of the next token
+        self.max_len = 0
+        self.first_key = None       # int32 [B]: first real key of each left-padded sample
+        self._hooked = False        # the attention hook has seen this layer's prompt pass
+        self._pending = False       # a decode token was handed out and not yet attended
+
+    # -- transformers.Cache protocol -----------------------------------------------------
+    def lazy_initialization(self, key_states, value_states):
+        self.dtype, self.device = key_states.dtype, key_states.device
+        self.is_initialized = True
+
+    def update(self, key_states, value_states, *args, **kwargs):
+        if key_states.shape[-2] != 1 or self.engine is None:
+            return self._prompt_pass(key_states, value_states)
+        if not self._hooked:
+            raise RuntimeError("FFACache: the model's attention does not go through the 'ffa' hook; "
+                               "call fastforwardattention_amd.hf.enable(model) first")
+        if self._pending:
+            raise RuntimeError("FFACache: the previous decode token of this layer was never attended")
+        if self.t >= self.max_len:
+            raise RuntimeError(f"FFACache: cache full ({self.max_len} slots = prompt + max_new_tokens)")
+        self._pending = True
+        setattr(key_states, _TAG, self)
+        return key_states, value_states
+
+    def get_seq_length(self) -> int:
+        return self.t
+
+    def get_mask_sizes(self, query_length: int):
+        return self.t + query_length, 0
+
+    def get_max_length(self) -> int:
+        return -1
+
+    def reset(self):
+        self.engine, self.t, self.max_len, self.first_key = None, 0, 0, None
+        self._hooked = self._pending = False
+
+    def _unsupported(self, *a, **k):
+        raise NotImplementedError("FFACache holds the reference's fixed-layout caches: no beam reordering, "
+                                  "cropping or batch reshaping (the reference disables cache_indir too)")
+
+    reorder_cache = crop = batch_repeat_interleave = batch_select_indices = offload = prefetch = _unsupported
+
+    # -- the two passes -------------------------------------------------------------------
+    def _prompt_pass(self, key_states, value_states):
+        if self.engine is not None:
+            raise NotImplementedError("FFACache: a second multi-token pass (chunked prefill, assisted decoding) "
+                                      "is not supported; the reference builds its caches from one prompt pass")
+        if not self.is_initialized:
+            self.lazy_initialization(key_states, value_states)
+        cls = self._engine_cls or _default_engine()
+        prompt_len = key_states.shape[-2]
+        self.max_len = prompt_len + self.max_new_tokens
+        self.engine = cls(key_states.contiguous(), value_states.to(key_states.dtype).contiguous(),
+                          self.max_len, self.use_default_kernel_launch)
+        self.t = prompt_len
+        setattr(key_states, _TAG, self)
+        return key_states, value_states
+
+    def note_prompt_mask(self, attention_mask):
+        """Left-padding offsets from the prompt pass's mask, as the reference takes them:
+        index of the first maximum of the last query row (modeling_opt.py:222)."""
+        self._hooked = True
+        if attention_mask is None:
+            self.first_key = None
+            return
+        row = attention_mask[:, :, -1, :]
+        if row.dtype == torch.bool:
+            row = row.to(torch.int8)
+        self.first_key = torch.max(row, dim=-1).indices.reshape(-1).to(torch.int32).contiguous()
+
+    def attend(self, query, key, value, scale: float):
+        """One decode step: [B,H,1,Dh] q/k/v -> [B,H,Dh]; appends k, v at slot t."""
+        if not self._pending:
+            raise RuntimeError("FFACache: attend() without a pending decode token")
+        dt = self.dtype
+        q, k, v = query.to(dt), key.to(dt), value.to(dt)
+        k_cache, v_cache = self.engine.get_cache()
+        if self.first_key is None:
+            out = self.engine.attention(q, k, v, k_cache, v_cache, float(scale), self.t, self.prob_thresh)
+        else:
+            out = self.engine.attention(q, k, v, k_cache, v_cache, float(scale), self.t, self.first_key,
+                                        self.prob_thresh)
+        self.t += 1
+        self._pending = False
+        return out
+
+
+class FFACache(Cache):
+    """`past_key_values` object that keeps every layer's keys and values inside a
+    `FastForwardAttn` (cache layouts [B,H,Dh/x,Lmax,x] / [B,H,Lmax,Dh], Lmax = prompt +
+    max_new_tokens).  `engine` replaces the `FastForwardAttn` class (same constructor and
+    methods); tests use it to run the bookkeeping without a GPU."""
+
+    def __init__(self, max_new_tokens: int, prob_thresh: float = 0.0,
+                 use_default_kernel_launch: bool = False, engine=None):
+        super().__init__(layer_class_to_replicate=functools.partial(
+            FFALayer, max_new_tokens, prob_thresh, use_default_kernel_launch, engine))
+
+    @classmethod
+    def from_env(cls, engine=None):
+        """The reference's switches (summarize.py:77-96; modeling_opt.py:196-199)."""
+        return cls(int(os.environ["max_tokens"]), float(os.environ.get("prob_thresh", "0")),
+                   int(os.environ.get("use_ffa_default_kl", "0")) == 1, engine)
+
+
+def enabled_by_env() -> bool:
+    """`use_ffa=1` in the environment, the reference's master switch (modeling_opt.py:196)."""
+    return int(os.environ.get("use_ffa", "0")) == 1
+
+
+# -- attention hooks --------------------------------------------------------------------------
+def _plain_attention(query, key, value, attention_mask, scaling):
+    """Ordinary masked softmax attention for the prompt pass; [B,H,Lq,Dh] in and out."""
+    w = torch.matmul(query, key.transpose(-1, -2)) * scaling
+    if attention_mask is not None:
+        w = w + attention_mask if attention_mask.dtype != torch.bool else w.masked_fill(~attention_mask, float("-inf"))
+    w = torch.softmax(w, dim=-1, dtype=torch.float32).to(value.dtype)
+    return torch.matmul(w, value)
+
+
+def ffa_attention_forward(module, query, key, value, attention_mask, scaling=None, dropout=0.0, **kwargs):
+    """Attention function for transformers' registry (`attn_implementation="ffa"`).
+    Returns ([B, Lq, H, Dh], None) like the built-in ones."""
+    if scaling is None:
+        scaling = query.shape[-1] ** -0.5
+    layer = getattr(key, _TAG, None)
+    if layer is not None and layer._pending:
+        return layer.attend(query, key, value, scaling).unsqueeze(1), None
+    if layer is not None:
+        layer.note_prompt_mask(attention_mask)
+    out = _plain_attention(query, key, value, attention_mask, scaling)
+    return out.transpose(1, 2).contiguous(), None
+
+
+def _gptj_attn(self, query, key, value, attention_mask=None, *rest):
+    """Replacement for GPTJAttention._attn (modeling_gptj.py:252-281): ([B,H,Lq,Dh], weights)."""
+    layer = getattr(key, _TAG, None)
+    if layer is not None and layer._pending:
+        return layer.attend(query, key, value, 1.0 / self.scale_attn).unsqueeze(2), None
+    if layer is not None:
+        layer.note_prompt_mask(attention_mask)
+    return self._ffa_original_attn(query, key, value, attention_mask, *rest)
+
+
+def register():
+    """Make `"ffa"` known to transformers' attention and mask registries (idempotent)."""
+    AttentionInterface.register(ATTN_NAME, ffa_attention_forward)
+    AttentionMaskInterface.register(ATTN_NAME, eager_mask)
+
+
+def enable(model):
+    """Route `model`'s decode steps through FastForwardAttn.  Pass an `FFACache` as
+    `past_key_values` afterwards; with any other cache the model behaves as before."""
+    register()
+    wrapped = 0
+    for mod in model.modules():
+        if type(mod).__name__.startswith("GPTJ") and hasattr(mod, "_attn") and hasattr(mod, "scale_attn"):
+            if not hasattr(mod, "_ffa_original_attn"):
+                mod._ffa_original_attn = mod._attn
+                mod._attn = types.MethodType(_gptj_attn, mod)
+            wrapped += 1
+    if wrapped == 0:
+        model._ffa_previous_attn = model.config._attn_implementation
+        model.config._attn_implementation = ATTN_NAME
+    return model
+
+
+def disable(model):
+    """Undo `enable`."""
+    for mod in model.modules():
+        if hasattr(mod, "_ffa_original_attn"):
+            del mod.__dict__["_attn"]          # the class's own method shows through again
+            del mod._ffa_original_attn
+    prev = getattr(model, "_ffa_previous_attn", None)
+    if prev is not None:
+        model.config._attn_implementation = prev
+        del model._ffa_previous_attn
+    return model
