@@ -342,6 +342,41 @@ def run_pruned_sweeps():
         torch.cuda.empty_cache()
 
 
+def run_init_cache_bench():
+    """Cache construction (ffa_init_cache_f16) at the BASELINE shapes: reads K, V [B,H,L,Dh] and
+    writes both cache layouts, 4*B*H*L*Dh*sizeof(T) bytes per call.  Source and destination sets
+    rotate so that no call finds its data in the 256 MB last-level cache."""
+    import torch
+    from fastforwardattention_amd import capi
+    lib = capi.load()
+    res = []
+    for name, (B, H, Dh, L, gen) in {"opt1.3b_b10": (10, 32, 64, 1000, 256), "gptj_b8": (8, 16, 256, 2000, 256),
+                                     "pruned_b16_8k": (16, 32, 64, 8192, 64)}.items():
+        Lmax = L + gen
+        per_call = 4 * B * H * L * Dh * 2
+        nsets = max(2, int(1.5e9 // per_call) + 1)
+        src = [(torch.randn(B, H, L, Dh, device="cuda:0", dtype=torch.float16),
+                torch.randn(B, H, L, Dh, device="cuda:0", dtype=torch.float16)) for _ in range(nsets)]
+        dst = [(torch.empty(B, H, Dh // 8, Lmax, 8, device="cuda:0", dtype=torch.float16),
+                torch.empty(B, H, Lmax, Dh, device="cuda:0", dtype=torch.float16)) for _ in range(nsets)]
+        sp = torch.cuda.current_stream().cuda_stream
+
+        def body(n):
+            for i in range(n):
+                (ks, vs), (kd, vd) = src[i % nsets], dst[i % nsets]
+                capi.check(lib.ffa_init_cache_f16(kd.data_ptr(), vd.data_ptr(), ks.data_ptr(), vs.data_ptr(),
+                                                  B, L, Lmax, Dh, H, sp), "ffa_init_cache_f16")
+        body(nsets)
+        reps = 4 * nsets
+        us = time_region(torch, lambda: body(reps)) * 1e3 / reps
+        res.append({"workload": name, "shape": [B, H, L, Dh], "max_len": Lmax, "bytes_per_call": per_call,
+                    "us_per_call": round(us, 2), "GBps": round(per_call / us / 1e3, 1),
+                    "hbm_frac": round(per_call / us / 1e3 / HBM_PEAK_GBS, 4)})
+        del src, dst
+        torch.cuda.empty_cache()
+    return {"kernel": "ffa_init_cache_kernel (cache construction, fp16)", "results": res}
+
+
 def run_suite(args):
     """Every BASELINE.json configuration that fits one GPU, one JSON object per line."""
     for name in ["opt1.3b_b10", "opt1.3b_b5", "opt1.3b_b2", "opt1.3b_b1", "gptj_b8",
@@ -360,6 +395,7 @@ def run_suite(args):
             import torch
             torch.cuda.empty_cache()
     run_pruned_sweeps()
+    print(json.dumps(run_init_cache_bench()), flush=True)
 
 
 def run_copy_calibration(mib=128, reps=40):
@@ -406,6 +442,7 @@ def main():
     ap.add_argument("--suite", action="store_true",
                     help="run every BASELINE configuration (tuned and default launch) and the pruned sweep; "
                          "one JSON line each instead of the single headline line")
+    ap.add_argument("--init-cache", action="store_true", help="only the cache-construction kernel at the BASELINE shapes")
     ap.add_argument("--pruned-sweep", action="store_true", help="only the pruned sweep (BASELINE configs[4])")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="run a plain 128 MiB copy kernel 40 times (reference for rocprofv3 --pmc FETCH_SIZE / "
@@ -429,6 +466,9 @@ def main():
         return
     if args.pruned_sweep:
         run_pruned_sweeps()
+        return
+    if args.init_cache:
+        print(json.dumps(run_init_cache_bench()))
         return
 
     plan_override = tuple(int(x) for x in args.plan.split(",")) if args.plan else None
