@@ -12,7 +12,8 @@ namespace ffa {
 constexpr int kTileKeys = 64;            // keys per wave tile (= wavefront size)
 constexpr int kMaxSplits = 128;          // upper bound on workgroups per (batch, head)
 constexpr int kMaxSplitWorkgroups = 16384;  // upper bound on workgroups of a split launch
-constexpr int kMaxDynamicLdsBytes = 160 * 1024 - 4096;  // gfx950: 160 KiB LDS per CU, minus statics
+constexpr int kMaxDynamicLdsBytes = 160 * 1024 - 20 * 1024;  // gfx950: 160 KiB LDS per CU, minus statics
+                                                             // (16 KiB of survivor queues at 16 waves)
 
 // Arguments of one decode step, after validation.
 struct DecodeArgs {

@@ -190,6 +190,77 @@ __device__ __forceinline__ float acquire(const float* p) {
 }
 
 // ---------------------------------------------------------------------------------------
+// Survivor queue of the pruning kernels.  A key that the rule drops must cost neither bytes
+// nor instructions, so the keys that survive are compacted, per wave, into an LDS queue of
+// two 64-entry blocks (weight + cache row each); a block is consumed as soon as it is full,
+// by the same V mapping as an ordinary tile: every lane active, every load a surviving row.
+// Entry n of the stream sits in block (n >> 6) & 1 at stage_slot(n & 63).
+struct SurvivorQueue {
+    float* w;          // this wave's 128 weights
+    int* row;          // this wave's 128 cache rows
+    unsigned total;    // survivors pushed so far (wave-uniform)
+};
+
+// P.V over one queue block holding `count` valid entries (64 unless it is the last one).
+template <typename T, int DH>
+__device__ __forceinline__ void pv_queue_block(float (&acc)[Elem<T>::X], const SurvivorQueue& q, int block,
+                                               int count, const char* vc_bh, const char* vnew, int tlen,
+                                               int lane) {
+    using G = Geo<T, DH>;
+    constexpr int NCH = G::NCH, LPR = G::LPR, RPI = G::RPI;
+    constexpr int VG = NCH < 8 ? NCH : 8;
+    const int rg = lane / LPR, dch = lane % LPR;
+    const float* pw = q.w + block * kWave + rg * NCH;
+    const int* pr = q.row + block * kWave + rg * NCH;
+#pragma unroll 1
+    for (int g = 0; g < NCH / VG; ++g) {
+        uint4 vv[VG];
+        float pj[VG];
+#pragma unroll
+        for (int j = 0; j < VG; ++j) {
+            const int n = (g * VG + j) * RPI + rg;  // entry number inside the block
+            pj[j] = 0.f;
+            vv[j] = make_uint4(0, 0, 0, 0);
+            if (n < count) {
+                const int r = pr[g * VG + j];
+                pj[j] = pw[g * VG + j];
+                vv[j] = ld16(r < tlen ? vc_bh + ((size_t)r * NCH + dch) * 16 : vnew + dch * 16);
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < VG; ++j) fma_chunk(acc, pj[j], vv[j], T{});
+    }
+}
+
+// Push this lane's key if it survives; consumes a block when one fills up.
+template <typename T, int DH>
+__device__ __forceinline__ void queue_push(float (&acc)[Elem<T>::X], SurvivorQueue& q, bool keep, float weight,
+                                           int key, const char* vc_bh, const char* vnew, int tlen, int lane) {
+    using G = Geo<T, DH>;
+    const unsigned long long mask = __builtin_amdgcn_ballot_w64(keep);
+    const unsigned before =
+        __builtin_amdgcn_mbcnt_hi((unsigned)(mask >> 32), __builtin_amdgcn_mbcnt_lo((unsigned)mask, 0u));
+    if (keep) {
+        const unsigned n = q.total + before;
+        const int slot = ((n >> 6) & 1) * kWave + stage_slot<G::NCH, G::RPI>(n & 63);
+        q.w[slot] = weight;
+        q.row[slot] = key;
+    }
+    const unsigned after = q.total + (unsigned)__builtin_popcountll(mask);
+    __builtin_amdgcn_wave_barrier();
+    if ((after >> 6) != (q.total >> 6))  // wave-uniform: a block has just been completed
+        pv_queue_block<T, DH>(acc, q, (q.total >> 6) & 1, kWave, vc_bh, vnew, tlen, lane);
+    q.total = after;
+    __builtin_amdgcn_wave_barrier();
+}
+
+template <typename T, int DH>
+__device__ __forceinline__ void queue_drain(float (&acc)[Elem<T>::X], SurvivorQueue& q, const char* vc_bh,
+                                            const char* vnew, int tlen, int lane) {
+    if (q.total & 63) pv_queue_block<T, DH>(acc, q, (q.total >> 6) & 1, q.total & 63, vc_bh, vnew, tlen, lane);
+}
+
+// ---------------------------------------------------------------------------------------
 // Sequence-split exact decode (p == 0).
 template <typename T, int DH, int NW>
 __global__ void __launch_bounds__(NW * 64) ffa_decode_split_kernel(const DecodeParams P) {
@@ -493,6 +564,8 @@ __global__ void __launch_bounds__(NW * 64) ffa_decode_wg_kernel(const DecodePara
     __shared__ float s_red[NW];
     __shared__ unsigned s_cnt[NW];
     __shared__ uint4 s_q[G::Q_LDS ? NCH : 1];
+    __shared__ float s_qw[NW][2 * kWave];
+    __shared__ int s_qr[NW][2 * kWave];
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int bh = blockIdx.x;
@@ -606,31 +679,38 @@ __global__ void __launch_bounds__(NW * 64) ffa_decode_wg_kernel(const DecodePara
         P.kept_count[bh] = tot;
     }
 
-    // ---- phase 3: P.V with the skip fused in ----
+    // ---- phase 3: P.V.  Pruned: only the surviving rows, compacted per wave ----
     const int rg = lane / LPR, dch = lane % LPR;
     float acc[X];
 #pragma unroll
     for (int e = 0; e < X; ++e) acc[e] = 0.f;
-    for (int tile = tile_lo + wave; tile < ntiles; tile += NW) {
+    if (pruned) {
+        SurvivorQueue sq = {s_qw[wave], s_qr[wave], 0u};
+        for (int tile = tile_lo + wave; tile < ntiles; tile += NW) {
+            const int key = tile * kWave + lane;
+            const float w = s_sc[key];
+            queue_push<T, DH>(acc, sq, w >= 0.f, w, key, vc_bh, vnew, tlen, lane);
+        }
+        queue_drain<T, DH>(acc, sq, vc_bh, vnew, tlen, lane);
+    } else {
+        for (int tile = tile_lo + wave; tile < ntiles; tile += NW) {
 #pragma unroll 1
-        for (int g = 0; g < NCH / VG; ++g) {
-            uint4 vv[VG];
-            float pj[VG];
+            for (int g = 0; g < NCH / VG; ++g) {
+                uint4 vv[VG];
+                float pj[VG];
 #pragma unroll
-            for (int j = 0; j < VG; ++j) {
-                const int row = tile * kWave + (g * VG + j) * RPI + rg;
-                pj[j] = s_sc[row];
-                const bool keep = pruned ? (pj[j] >= 0.f) : (row <= tlen);
-                vv[j] = make_uint4(0, 0, 0, 0);
-                if (keep) {
-                    const char* vp = row < tlen ? vc_bh + ((size_t)row * NCH + dch) * 16 : vnew + dch * 16;
-                    vv[j] = ld16(vp);
-                } else {
-                    pj[j] = 0.f;
+                for (int j = 0; j < VG; ++j) {
+                    // Unconditional loads (rows past the end re-read the new token with
+                    // weight 0): a load under a branch would have to be waited for at the
+                    // join, one round trip per row.
+                    const int row = tile * kWave + (g * VG + j) * RPI + rg;
+                    pj[j] = row <= tlen ? s_sc[row] : 0.f;
+                    const int r = min(row, tlen);
+                    vv[j] = ld16(r < tlen ? vc_bh + ((size_t)r * NCH + dch) * 16 : vnew + dch * 16);
                 }
-            }
 #pragma unroll
-            for (int j = 0; j < VG; ++j) fma_chunk(acc, pj[j], vv[j], T{});
+                for (int j = 0; j < VG; ++j) fma_chunk(acc, pj[j], vv[j], T{});
+            }
         }
     }
 
@@ -734,10 +814,10 @@ __global__ void __launch_bounds__(NW * 64) ffa_scores_kernel(const DecodeParams 
 template <typename T, int DH, int NW>
 __global__ void __launch_bounds__(NW * 64) ffa_pruned_pv_kernel(const DecodeParams P) {
     using G = Geo<T, DH>;
-    constexpr int X = G::X, NCH = G::NCH, LPR = G::LPR, RPI = G::RPI;
-    constexpr int VG = NCH < 8 ? NCH : 8;
+    constexpr int X = G::X, LPR = G::LPR;
     constexpr int NT = NW * 64;
-    __shared__ float s_p[NW][kWave];
+    __shared__ float s_qw[NW][2 * kWave];
+    __shared__ int s_qr[NW][2 * kWave];
     __shared__ float s_acc[NW][DH];
     __shared__ unsigned s_cnt[NW];
     __shared__ int s_last;
@@ -787,12 +867,12 @@ __global__ void __launch_bounds__(NW * 64) ffa_pruned_pv_kernel(const DecodePara
     float thr_key = 0.f;
     if (pruned) (void)round_prob(P.p * inv, T{}, &thr_key);
 
-    // ---- own tiles: weights (one key per lane) -> LDS stage -> surviving V rows ----
-    const int rg = lane / LPR, dch = lane % LPR;
+    // ---- own tiles: weights (one key per lane) -> survivor queue -> surviving V rows ----
     float acc[X];
 #pragma unroll
     for (int e = 0; e < X; ++e) acc[e] = 0.f;
     unsigned kept = 0;
+    SurvivorQueue sq = {s_qw[wave], s_qr[wave], 0u};
     for (int tile = tile_lo + wave; tile < tile_hi; tile += NW) {
         const int key = tile * kWave + lane;
         const float sr = sr_next;
@@ -813,31 +893,9 @@ __global__ void __launch_bounds__(NW * 64) ffa_pruned_pv_kernel(const DecodePara
             kept += drop ? 0u : 1u;
             if (P.skip_mask) P.skip_mask[(size_t)bh * P.Lmax + key] = drop ? 1 : 0;
         }
-        __builtin_amdgcn_wave_barrier();
-        s_p[wave][stage_slot<NCH, RPI>(lane)] = drop ? -1.f : w;
-        __builtin_amdgcn_wave_barrier();
-        const float* pst = &s_p[wave][rg * NCH];
-#pragma unroll 1
-        for (int g = 0; g < NCH / VG; ++g) {
-            uint4 vv[VG];
-            float pj[VG];
-#pragma unroll
-            for (int j = 0; j < VG; ++j) {
-                const int row = tile * kWave + (g * VG + j) * RPI + rg;
-                pj[j] = pst[g * VG + j];
-                vv[j] = make_uint4(0, 0, 0, 0);
-                if (pj[j] >= 0.f) {
-                    const char* vp = row < tlen ? vc_bh + ((size_t)row * NCH + dch) * 16 : vnew + dch * 16;
-                    vv[j] = ld16(vp);
-                } else {
-                    pj[j] = 0.f;
-                }
-            }
-#pragma unroll
-            for (int j = 0; j < VG; ++j) fma_chunk(acc, pj[j], vv[j], T{});
-        }
-        __builtin_amdgcn_wave_barrier();
+        queue_push<T, DH>(acc, sq, !drop, w, key, vc_bh, vnew, tlen, lane);
     }
+    queue_drain<T, DH>(acc, sq, vc_bh, vnew, tlen, lane);
     if (P.skip_mask && split == 0)  // keys of fully masked leading tiles are dropped too
         for (int i = tid; i < min(tile_first * kWave, tlen); i += NT) P.skip_mask[(size_t)bh * P.Lmax + i] = 1;
 

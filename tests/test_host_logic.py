@@ -140,7 +140,7 @@ def test_planner_consistency(prec, Dh):
                     assert plan.threads_per_key == 1 and plan.keys_per_wave == 64
                     assert plan.waves_per_wg in (1, 2, 4, 8, 16)
                     assert plan.n_splits * plan.tiles_per_split >= ntiles      # every key covered
-                    fits_lds = ntiles * 64 * 4 <= 156 * 1024
+                    fits_lds = ntiles * 64 * 4 <= 140 * 1024
                     if use_default:
                         assert plan.n_splits == 1
                         assert plan.kind == (capi.FFA_LAUNCH_WORKGROUP if fits_lds else capi.FFA_LAUNCH_TWO_PASS)
