@@ -218,14 +218,12 @@ __device__ __forceinline__ void pv_queue_block(float (&acc)[Elem<T>::X], const S
         float pj[VG];
 #pragma unroll
         for (int j = 0; j < VG; ++j) {
+            // Loads are unconditional (a load under a branch is waited for at the join, one
+            // round trip per row): entries past `count` re-read the new token with weight 0.
             const int n = (g * VG + j) * RPI + rg;  // entry number inside the block
-            pj[j] = 0.f;
-            vv[j] = make_uint4(0, 0, 0, 0);
-            if (n < count) {
-                const int r = pr[g * VG + j];
-                pj[j] = pw[g * VG + j];
-                vv[j] = ld16(r < tlen ? vc_bh + ((size_t)r * NCH + dch) * 16 : vnew + dch * 16);
-            }
+            const int r = n < count ? pr[g * VG + j] : tlen;
+            pj[j] = n < count ? pw[g * VG + j] : 0.f;
+            vv[j] = ld16(r < tlen ? vc_bh + ((size_t)r * NCH + dch) * 16 : vnew + dch * 16);
         }
 #pragma unroll
         for (int j = 0; j < VG; ++j) fma_chunk(acc, pj[j], vv[j], T{});
@@ -960,33 +958,46 @@ __global__ void __launch_bounds__(NW * 64) ffa_pruned_pv_kernel(const DecodePara
 
 // ---------------------------------------------------------------------------------------
 // Cache construction (attention.cu:1556-1609).  One workgroup moves a tile of TK keys of
-// one (b,h): coalesced row reads [64 keys x Dh] -> LDS -> coalesced 1 KiB chunk-row writes
-// for K; V is a straight strided copy.
+// one (b,h), TK*NCH 16-byte chunks each of K and V: coalesced row reads [TK keys x Dh] -> LDS
+// -> coalesced chunk-row writes (TK x 16 B contiguous) for K; V is a straight copy.  All
+// loads of a thread are issued before anything is stored (indices past the end are clamped,
+// so no load sits under a branch).
 template <int NCH, int TK>
 __global__ void __launch_bounds__(256) ffa_init_cache_kernel(uint4* __restrict__ k_dst,
                                                              uint4* __restrict__ v_dst,
                                                              const uint4* __restrict__ k_src,
                                                              const uint4* __restrict__ v_src,
                                                              int L, int Lmax) {
+    constexpr int PER = TK * NCH / 256;  // chunks per thread, of K and of V
+    static_assert(TK * NCH % 256 == 0 && PER >= 1, "tile must divide over the workgroup");
     __shared__ uint4 s_tile[NCH * (TK + 1)];  // [chunk][key], one chunk of padding per row
     const int bh = blockIdx.y;
     const int l0 = blockIdx.x * TK;
-    const int nkeys = min(TK, L - l0);
+    const int n = min(TK, L - l0) * NCH;  // chunks of this tile, >= NCH
     const uint4* ks = k_src + ((size_t)bh * L + l0) * NCH;
     const uint4* vs = v_src + ((size_t)bh * L + l0) * NCH;
-    uint4* kd = k_dst + (size_t)bh * Lmax * NCH;
+    uint4* kd = k_dst + (size_t)bh * Lmax * NCH + l0;
     uint4* vd = v_dst + ((size_t)bh * Lmax + l0) * NCH;
-    // V: contiguous copy of nkeys*NCH chunks.
-    for (int i = threadIdx.x; i < nkeys * NCH; i += 256) vd[i] = vs[i];
-    // K: read [key][chunk] (contiguous), write [chunk][key].
-    for (int i = threadIdx.x; i < nkeys * NCH; i += 256) {
-        const int key = i / NCH, c = i % NCH;
-        s_tile[c * (TK + 1) + key] = ks[i];
+    uint4 kv[PER], vv[PER];
+#pragma unroll
+    for (int j = 0; j < PER; ++j) {
+        const int i = min((int)threadIdx.x + j * 256, n - 1);
+        kv[j] = ks[i];
+        vv[j] = vs[i];
+    }
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int j = 0; j < PER; ++j) {
+        const int i = threadIdx.x + j * 256;
+        if (i < n) vd[i] = vv[j];                              // V: contiguous copy
+        s_tile[(i % NCH) * (TK + 1) + i / NCH] = kv[j];        // K: [key][chunk] -> [chunk][key]
     }
     __syncthreads();
-    for (int i = threadIdx.x; i < TK * NCH; i += 256) {
+#pragma unroll
+    for (int j = 0; j < PER; ++j) {
+        const int i = threadIdx.x + j * 256;
         const int c = i / TK, key = i % TK;
-        if (key < nkeys) kd[(size_t)c * Lmax + l0 + key] = s_tile[c * (TK + 1) + key];
+        if (key * NCH < n) kd[(size_t)c * Lmax + key] = s_tile[c * (TK + 1) + key];
     }
 }
 
@@ -1113,7 +1124,13 @@ int launch_decode(const DecodeArgs& a, const ffa_launch_plan& plan, const Worksp
 int launch_init_cache(int precision, void* k_dst, void* v_dst, const void* k_src,
                       const void* v_src, int B, int H, int L, int Lmax, int Dh, void* stream) {
     const int nch = Dh * (precision / 8) / 16;
-    const int tk = nch <= 32 ? 64 : 32;  // keeps the LDS tile under 64 KiB
+    if (nch != 8 && nch != 16 && nch != 32 && nch != 64) return FFA_ERR_HEAD_DIM;
+    if (L <= 0) return FFA_OK;
+    // 512 chunks (8 KiB of K, 8 KiB of V) per workgroup: measured against 1024 / 2048 / 4096,
+    // the small tile wins at every shape -- many resident workgroups hide the latency better
+    // than more loads per thread do.
+    constexpr int kIc = 512;
+    const int tk = kIc / nch;
     const dim3 grid((unsigned)((L + tk - 1) / tk), (unsigned)(B * H));
     hipStream_t st = reinterpret_cast<hipStream_t>(stream);
     auto kd = reinterpret_cast<uint4*>(k_dst);
@@ -1121,10 +1138,10 @@ int launch_init_cache(int precision, void* k_dst, void* v_dst, const void* k_src
     auto ks = reinterpret_cast<const uint4*>(k_src);
     auto vs = reinterpret_cast<const uint4*>(v_src);
     switch (nch) {
-        case 8: hipLaunchKernelGGL((ffa_init_cache_kernel<8, 64>), grid, dim3(256), 0, st, kd, vd, ks, vs, L, Lmax); break;
-        case 16: hipLaunchKernelGGL((ffa_init_cache_kernel<16, 64>), grid, dim3(256), 0, st, kd, vd, ks, vs, L, Lmax); break;
-        case 32: hipLaunchKernelGGL((ffa_init_cache_kernel<32, 64>), grid, dim3(256), 0, st, kd, vd, ks, vs, L, Lmax); break;
-        case 64: hipLaunchKernelGGL((ffa_init_cache_kernel<64, 32>), grid, dim3(256), 0, st, kd, vd, ks, vs, L, Lmax); break;
+        case 8: hipLaunchKernelGGL((ffa_init_cache_kernel<8, kIc / 8>), grid, dim3(256), 0, st, kd, vd, ks, vs, L, Lmax); break;
+        case 16: hipLaunchKernelGGL((ffa_init_cache_kernel<16, kIc / 16>), grid, dim3(256), 0, st, kd, vd, ks, vs, L, Lmax); break;
+        case 32: hipLaunchKernelGGL((ffa_init_cache_kernel<32, kIc / 32>), grid, dim3(256), 0, st, kd, vd, ks, vs, L, Lmax); break;
+        case 64: hipLaunchKernelGGL((ffa_init_cache_kernel<64, kIc / 64>), grid, dim3(256), 0, st, kd, vd, ks, vs, L, Lmax); break;
         default: return FFA_ERR_HEAD_DIM;
     }
     return check_launch();
