@@ -58,7 +58,7 @@ def algorithmic_bytes(B, H, Dh, t, elem=2):
 
 
 class Workload:
-    def __init__(self, name, use_default=False, plan_override=None):
+    def __init__(self, name, use_default=False, plan_override=None, layers=None):
         import torch
         from fastforwardattention_amd import capi
         self.torch, self.capi = torch, capi
@@ -66,7 +66,7 @@ class Workload:
         self.name = name
         w = WORKLOADS[name]
         self.B, self.H, self.Dh = w["B"], w["H"], w["Dh"]
-        self.prompt, self.gen, self.scale, self.layers = w["prompt"], w["gen"], w["scale"], w["layers"]
+        self.prompt, self.gen, self.scale, self.layers = w["prompt"], w["gen"], w["scale"], layers or w["layers"]
         self.Lmax = self.prompt + self.gen
         self.use_default = use_default
         self.plan_override = plan_override
@@ -222,10 +222,23 @@ def cpu_baseline(wl, budget_s=15.0, max_steps=64):
     mean_s = sum(times) / len(times)
     t_mid = L + 3 + len(times) // 2
     gbs = algorithmic_bytes(B, H, Dh, t_mid, elem=4) / mean_s / 1e9
+    # the same steps on one thread (a few of them: bounded at ~3 s)
+    nthreads = torch.get_num_threads()
+    torch.set_num_threads(1)
+    one, t0 = [], time.perf_counter()
+    while len(one) < 8 and (time.perf_counter() - t0) < 3.0:
+        q, k, v = toks[len(one) % 8]
+        s = time.perf_counter()
+        base.attention(q, k, v, wl.scale, L + 3 + len(times) + len(one))
+        one.append(time.perf_counter() - s)
+    torch.set_num_threads(nthreads)
+    one_s = sum(one) / len(one)
     return {
         "value": round(gbs, 3), "unit": "GB/s", "cores": torch.get_num_threads(),
         "host_cpus": os.cpu_count(), "kind": "port",
         "us_per_step": round(mean_s * 1e6, 1),
+        "one_thread": {"value": round(algorithmic_bytes(B, H, Dh, t_mid, elem=4) / one_s / 1e9, 3), "unit": "GB/s",
+                       "us_per_step": round(one_s * 1e6, 1), "steps": len(one)},
         "sample": (f"{len(times)} decode steps of {wl.name} (one layer, t={L + 3}..{L + 2 + len(times)}), "
                    "fp32 torch bmm/softmax/bmm over a pre-allocated cache; bytes counted at 4 B/element"),
     }
@@ -436,6 +449,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=240)
     ap.add_argument("--workload", default="opt1.3b_b10", choices=sorted(WORKLOADS))
     ap.add_argument("--default-launch", action="store_true", help="use_default_kernel_launch=True")
+    ap.add_argument("--layers", type=int, default=None,
+                    help="independent layer caches used round-robin (default: the model's layer count; 1 = a single "
+                         "cache, which at the headline shape stays resident in the 256 MB last-level cache)")
     ap.add_argument("--plan", default=None, help="kind,waves,tiles_per_split[,combine[,whole_heads]] (kind: 0 workgroup, 1 split; combine: 0 fused, 1 kernel)")
     ap.add_argument("--legs", default="graph,capi,ext", help="comma list of graph,capi,ext")
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -472,7 +488,7 @@ def main():
         return
 
     plan_override = tuple(int(x) for x in args.plan.split(",")) if args.plan else None
-    wl = Workload(args.workload, use_default=args.default_launch, plan_override=plan_override)
+    wl = Workload(args.workload, use_default=args.default_launch, plan_override=plan_override, layers=args.layers)
     steps, warmup = args.steps, args.warmup
     legs = [x for x in args.legs.split(",") if x]
     mean_b = wl.mean_bytes(steps)

@@ -259,6 +259,136 @@ __device__ __forceinline__ void queue_drain(float (&acc)[Elem<T>::X], SurvivorQu
 }
 
 // ---------------------------------------------------------------------------------------
+// End of a split-launch workgroup: every wave arrives with its own running (max, sum) and
+// its unnormalised accumulators.  Merges the lanes of a wave, the waves of the workgroup
+// (LDS), then writes the output (whole pair) or publishes a partial that the last piece of
+// the pair to arrive merges.
+template <typename T, int DH, int NW>
+__device__ __forceinline__ void finish_piece(const DecodeParams& P, int bh, int split, int n_splits,
+                                             float (&acc)[Elem<T>::X], float m_run, float l_run,
+                                             float (*s_acc)[DH], float* s_m, float* s_l, int* s_last_p) {
+    using G = Geo<T, DH>;
+    constexpr int X = G::X, LPR = G::LPR;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    int& s_last = *s_last_p;
+#ifdef FFA_TRACE
+    unsigned long long* ffa_row = nullptr;
+    if (P.trace) ffa_row = P.trace + (size_t)__builtin_amdgcn_readfirstlane(blockIdx.x * NW + wave) * 16;
+#endif
+    FFA_TP(3);
+    // ---- merge inside the wave: the RPI row groups (lanes with equal lane % LPR) ----
+#pragma unroll
+    for (int off = LPR; off < kWave; off <<= 1) {
+#pragma unroll
+        for (int e = 0; e < X; ++e) acc[e] += __shfl_xor(acc[e], off);
+    }
+    // ---- merge the waves of this workgroup (LDS): DH floats + (max, sum) per wave ----
+    l_run = wave_sum(l_run);
+    if (lane == 0) { s_m[wave] = m_run; s_l[wave] = l_run; }
+    if (lane < LPR) {
+#pragma unroll
+        for (int e = 0; e < X; ++e) s_acc[wave][lane * X + e] = acc[e];
+    }
+    __syncthreads();
+
+    float M = -INFINITY;
+#pragma unroll
+    for (int w = 0; w < NW; ++w) M = fmaxf(M, s_m[w]);
+    float L = 0.f;
+    float wgt[NW];
+#pragma unroll
+    for (int w = 0; w < NW; ++w) {
+        wgt[w] = (s_m[w] == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(s_m[w] - M);
+        L += wgt[w] * s_l[w];
+    }
+
+    T* out = reinterpret_cast<T*>(P.out) + (size_t)bh * DH;
+    // Partials of split pairs: slot (bh - n_whole) of the workspace.
+    const size_t slot0 = (size_t)(bh - P.n_whole) * P.n_splits;
+    float* wa = P.ws_acc + (slot0 + split) * DH;
+    for (int d = tid; d < DH; d += NW * 64) {
+        float o = 0.f;
+#pragma unroll
+        for (int w = 0; w < NW; ++w) o += wgt[w] * s_acc[w][d];
+        if (n_splits == 1) store_out(out, d, L > 0.f ? o / L : 0.f);
+        else if (P.combine == FFA_COMBINE_FUSED) publish(&wa[d], o);
+        else wa[d] = o;
+    }
+    if (n_splits == 1) return;
+    if (P.combine != FFA_COMBINE_FUSED) {
+        // A second kernel merges: plain stores would do, the kernel boundary publishes them.
+        if (tid == 0) {
+            float* ml = P.ws_ml + (slot0 + split) * 2;
+            ml[0] = M;
+            ml[1] = L;
+        }
+        return;
+    }
+
+    // ---- publish the partial; the last workgroup to arrive merges all splits ----
+    // No device-scope fence here: on this part such a fence writes back / invalidates a
+    // whole L2 and costs far more than the kernel itself.  Instead every word that crosses
+    // workgroups is moved with device-scope atomic accesses, which the hardware performs
+    // at the level all XCDs share, so nothing needs flushing.  Order: each thread's
+    // published stores are complete before the workgroup barrier (the barrier waits for
+    // outstanding memory operations), the arrival counter is bumped after it, and the
+    // merging workgroup reads the partials only after it has seen the final count.
+    if (tid == 0) {
+        float* ml = P.ws_ml + (slot0 + split) * 2;
+        publish(&ml[0], M);
+        publish(&ml[1], L);
+    }
+    FFA_TP(4);
+    __syncthreads();
+    FFA_TP(5);
+    if (tid == 0) {
+        const unsigned prev =
+            __hip_atomic_fetch_add(&P.ws_cnt[bh], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        s_last = (prev == (unsigned)(n_splits - 1));
+    }
+    __syncthreads();
+    FFA_TP(6);
+    if (!s_last) return;
+
+    // Merge: all loads of a batch of splits are issued before any is consumed.
+    const float* ml = P.ws_ml + slot0 * 2;
+    constexpr int MB = 8;
+    for (int d = tid; d < DH; d += NW * 64) {
+        float Mg = -INFINITY, o = 0.f, Lg = 0.f;
+        for (int s0 = 0; s0 < n_splits; s0 += MB) {
+            float ms[MB], ls[MB], as[MB];
+#pragma unroll
+            for (int j = 0; j < MB; ++j) {
+                const int sj = min(s0 + j, n_splits - 1);
+                ms[j] = acquire(&ml[2 * sj]);
+                ls[j] = acquire(&ml[2 * sj + 1]);
+                as[j] = acquire(&P.ws_acc[(slot0 + sj) * DH + d]);
+            }
+            float Mb = Mg;
+#pragma unroll
+            for (int j = 0; j < MB; ++j)
+                if (s0 + j < n_splits) Mb = fmaxf(Mb, ms[j]);
+            const float rescale = (Mg == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(Mg - Mb);
+            o *= rescale;
+            Lg *= rescale;
+#pragma unroll
+            for (int j = 0; j < MB; ++j) {
+                if (s0 + j < n_splits && ms[j] != -INFINITY) {
+                    const float w = __builtin_amdgcn_exp2f(ms[j] - Mb);
+                    Lg += w * ls[j];
+                    o += w * as[j];
+                }
+            }
+            Mg = Mb;
+        }
+        store_out(out, d, Lg > 0.f ? o / Lg : 0.f);
+    }
+    FFA_TP(7);
+    // Ready for the next launch on this stream (kernel boundaries order this store).
+    if (tid == 0) __hip_atomic_store(&P.ws_cnt[bh], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// ---------------------------------------------------------------------------------------
 // Sequence-split exact decode (p == 0).
 template <typename T, int DH, int NW>
 __global__ void __launch_bounds__(NW * 64) ffa_decode_split_kernel(const DecodeParams P) {
@@ -412,117 +542,7 @@ __global__ void __launch_bounds__(NW * 64) ffa_decode_split_kernel(const DecodeP
     }
     if (appends) new_token_store<NCH>(new_tok, kc_bh, vc_bh, tlen, P.Lmax, lane);
 
-    FFA_TP(3);
-    // ---- merge inside the wave: the RPI row groups (lanes with equal lane % LPR) ----
-#pragma unroll
-    for (int off = LPR; off < kWave; off <<= 1) {
-#pragma unroll
-        for (int e = 0; e < X; ++e) acc[e] += __shfl_xor(acc[e], off);
-    }
-    // ---- merge the waves of this workgroup (LDS): DH floats + (max, sum) per wave ----
-    l_run = wave_sum(l_run);
-    if (lane == 0) { s_m[wave] = m_run; s_l[wave] = l_run; }
-    if (lane < LPR) {
-#pragma unroll
-        for (int e = 0; e < X; ++e) s_acc[wave][lane * X + e] = acc[e];
-    }
-    __syncthreads();
-
-    float M = -INFINITY;
-#pragma unroll
-    for (int w = 0; w < NW; ++w) M = fmaxf(M, s_m[w]);
-    float L = 0.f;
-    float wgt[NW];
-#pragma unroll
-    for (int w = 0; w < NW; ++w) {
-        wgt[w] = (s_m[w] == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(s_m[w] - M);
-        L += wgt[w] * s_l[w];
-    }
-
-    T* out = reinterpret_cast<T*>(P.out) + (size_t)bh * DH;
-    // Partials of split pairs: slot (bh - n_whole) of the workspace.
-    const size_t slot0 = (size_t)(bh - P.n_whole) * P.n_splits;
-    float* wa = P.ws_acc + (slot0 + split) * DH;
-    for (int d = tid; d < DH; d += NW * 64) {
-        float o = 0.f;
-#pragma unroll
-        for (int w = 0; w < NW; ++w) o += wgt[w] * s_acc[w][d];
-        if (n_splits == 1) store_out(out, d, L > 0.f ? o / L : 0.f);
-        else if (P.combine == FFA_COMBINE_FUSED) publish(&wa[d], o);
-        else wa[d] = o;
-    }
-    if (n_splits == 1) return;
-    if (P.combine != FFA_COMBINE_FUSED) {
-        // A second kernel merges: plain stores would do, the kernel boundary publishes them.
-        if (tid == 0) {
-            float* ml = P.ws_ml + (slot0 + split) * 2;
-            ml[0] = M;
-            ml[1] = L;
-        }
-        return;
-    }
-
-    // ---- publish the partial; the last workgroup to arrive merges all splits ----
-    // No device-scope fence here: on this part such a fence writes back / invalidates a
-    // whole L2 and costs far more than the kernel itself.  Instead every word that crosses
-    // workgroups is moved with device-scope atomic accesses, which the hardware performs
-    // at the level all XCDs share, so nothing needs flushing.  Order: each thread's
-    // published stores are complete before the workgroup barrier (the barrier waits for
-    // outstanding memory operations), the arrival counter is bumped after it, and the
-    // merging workgroup reads the partials only after it has seen the final count.
-    if (tid == 0) {
-        float* ml = P.ws_ml + (slot0 + split) * 2;
-        publish(&ml[0], M);
-        publish(&ml[1], L);
-    }
-    FFA_TP(4);
-    __syncthreads();
-    FFA_TP(5);
-    if (tid == 0) {
-        const unsigned prev =
-            __hip_atomic_fetch_add(&P.ws_cnt[bh], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        s_last = (prev == (unsigned)(n_splits - 1));
-    }
-    __syncthreads();
-    FFA_TP(6);
-    if (!s_last) return;
-
-    // Merge: all loads of a batch of splits are issued before any is consumed.
-    const float* ml = P.ws_ml + slot0 * 2;
-    constexpr int MB = 8;
-    for (int d = tid; d < DH; d += NW * 64) {
-        float Mg = -INFINITY, o = 0.f, Lg = 0.f;
-        for (int s0 = 0; s0 < n_splits; s0 += MB) {
-            float ms[MB], ls[MB], as[MB];
-#pragma unroll
-            for (int j = 0; j < MB; ++j) {
-                const int sj = min(s0 + j, n_splits - 1);
-                ms[j] = acquire(&ml[2 * sj]);
-                ls[j] = acquire(&ml[2 * sj + 1]);
-                as[j] = acquire(&P.ws_acc[(slot0 + sj) * DH + d]);
-            }
-            float Mb = Mg;
-#pragma unroll
-            for (int j = 0; j < MB; ++j)
-                if (s0 + j < n_splits) Mb = fmaxf(Mb, ms[j]);
-            const float rescale = (Mg == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(Mg - Mb);
-            o *= rescale;
-            Lg *= rescale;
-#pragma unroll
-            for (int j = 0; j < MB; ++j) {
-                if (s0 + j < n_splits && ms[j] != -INFINITY) {
-                    const float w = __builtin_amdgcn_exp2f(ms[j] - Mb);
-                    Lg += w * ls[j];
-                    o += w * as[j];
-                }
-            }
-            Mg = Mb;
-        }
-        store_out(out, d, Lg > 0.f ? o / Lg : 0.f);
-    }
-    FFA_TP(7);
-    // Ready for the next launch on this stream (kernel boundaries order this store).
-    if (tid == 0) __hip_atomic_store(&P.ws_cnt[bh], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    finish_piece<T, DH, NW>(P, bh, split, n_splits, acc, m_run, l_run, s_acc, s_m, s_l, &s_last);
 }
 
 // Merge kernel of FFA_COMBINE_KERNEL: one wave per split (b,h) pair, log-sum-exp over its
