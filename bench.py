@@ -43,6 +43,7 @@ WORKLOADS = {
     "opt1.3b_b5": dict(B=5, H=32, Dh=64, prompt=1000, gen=256, scale=0.125, layers=24),
     "opt1.3b_b2": dict(B=2, H=32, Dh=64, prompt=1000, gen=256, scale=0.125, layers=24),
     "opt1.3b_b1": dict(B=1, H=32, Dh=64, prompt=1000, gen=256, scale=0.125, layers=24),
+    "opt2.7b_b10": dict(B=10, H=32, Dh=80, prompt=1000, gen=256, scale=80 ** -0.5, layers=32),
     "gptj_b8": dict(B=8, H=16, Dh=256, prompt=2000, gen=256, scale=0.0625, layers=8),
     "long_b1_16k": dict(B=1, H=32, Dh=64, prompt=16384 - 128, gen=128, scale=0.125, layers=24),
     "long_b1_8k": dict(B=1, H=32, Dh=64, prompt=8192 - 128, gen=128, scale=0.125, layers=24),
@@ -392,7 +393,7 @@ def run_init_cache_bench():
 
 def run_suite(args):
     """Every BASELINE.json configuration that fits one GPU, one JSON object per line."""
-    for name in ["opt1.3b_b10", "opt1.3b_b5", "opt1.3b_b2", "opt1.3b_b1", "gptj_b8",
+    for name in ["opt1.3b_b10", "opt1.3b_b5", "opt1.3b_b2", "opt1.3b_b1", "opt2.7b_b10", "gptj_b8",
                  "long_b1_1k", "long_b1_2k", "long_b1_4k", "long_b1_8k", "long_b1_16k"]:
         for use_default in (False, True):
             wl = Workload(name, use_default=use_default)

@@ -14,7 +14,7 @@ bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) ==
 
 int validate_decode(const DecodeArgs& a) {
     if (a.precision != FFA_PRECISION_F16 && a.precision != FFA_PRECISION_F32) return FFA_ERR_DTYPE;
-    if (a.Dh != 64 && a.Dh != 128 && a.Dh != 256) return FFA_ERR_HEAD_DIM;
+    if (a.Dh != 64 && a.Dh != 80 && a.Dh != 128 && a.Dh != 256) return FFA_ERR_HEAD_DIM;
     if (a.B <= 0 || a.H <= 0 || a.Lmax <= 0) return FFA_ERR_SHAPE;
     if ((long long)a.B * a.H > (1ll << 24)) return FFA_ERR_SHAPE;
     if (a.t < 0 || a.t >= a.Lmax) return FFA_ERR_TIMESTEP;
@@ -82,7 +82,7 @@ int run_decode(const DecodeArgs& a, const ffa_launch_plan* user_plan, void* work
 
 int run_init_cache(int precision, void* k_dst, void* v_dst, const void* k_src, const void* v_src,
                    int B, int L, int Lmax, int Dh, int H, void* stream) {
-    if (Dh != 64 && Dh != 128 && Dh != 256) return FFA_ERR_HEAD_DIM;
+    if (Dh != 64 && Dh != 80 && Dh != 128 && Dh != 256) return FFA_ERR_HEAD_DIM;
     if (B <= 0 || H <= 0 || L < 0 || Lmax <= 0 || L > Lmax) return FFA_ERR_SHAPE;
     if (!k_dst || !v_dst) return FFA_ERR_NULL_POINTER;
     if (L == 0) return FFA_OK;
@@ -103,7 +103,7 @@ const char* ffa_status_string(int status) {
         case FFA_OK: return "ok";
         case FFA_ERR_NULL_POINTER: return "a required pointer is NULL";
         case FFA_ERR_DTYPE: return "unsupported precision (expected 16 or 32)";
-        case FFA_ERR_HEAD_DIM: return "unsupported head dimension (expected 64, 128 or 256)";
+        case FFA_ERR_HEAD_DIM: return "unsupported head dimension (expected 64, 80, 128 or 256)";
         case FFA_ERR_SHAPE: return "invalid batch, head or sequence size";
         case FFA_ERR_TIMESTEP: return "timestep outside [0, max_seq_len)";
         case FFA_ERR_ALIGNMENT: return "pointer is not 16-byte aligned";

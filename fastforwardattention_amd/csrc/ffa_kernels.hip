@@ -154,7 +154,7 @@ __device__ __forceinline__ float tile_qk(const char* kc_bh, const char* knew, in
     const bool cached = key < tlen;
     const char* kp = cached ? kc_bh + (size_t)key * 16 : knew;
     const size_t kstr = cached ? (size_t)Lmax * 16 : 16;
-    constexpr int CG = NCH < 8 ? NCH : 8;
+    constexpr int CG = NCH % 8 == 0 ? 8 : 10;
     float s = 0.f;
 #pragma unroll 2
     for (int g = 0; g < NCH / CG; ++g) {
@@ -169,17 +169,24 @@ template <typename T, int DH>
 struct Geo {
     static constexpr int X = Elem<T>::X;      // elements per 16 B
     static constexpr int NCH = DH / X;        // 16-byte chunks per key / per V row
-    static constexpr int LPR = NCH;           // lanes per V row
+    // Lanes per V row: the chunk count rounded up to a power of two (Dh = 80: 10 chunks on
+    // 16 lanes, the upper 6 repeat the last chunk and are never stored).
+    static constexpr int LPR = NCH <= 8 ? 8 : NCH <= 16 ? 16 : NCH <= 32 ? 32 : 64;
     static constexpr int RPI = kWave / LPR;   // V rows per load instruction
+    static constexpr int NVL = LPR;           // V load instructions per 64-key tile (= 64 / RPI)
+    static constexpr int ROWW = LPR * X;      // accumulator floats per row group across the wave
+    static constexpr int CG = NCH % 8 == 0 ? 8 : 10;  // K loads in flight per group
+    static constexpr int VG = 8;                      // V loads in flight per group
     static constexpr bool Q_LDS = NCH > 16;   // q kept in LDS when it would not fit SGPR/VGPRs
     static constexpr int QREG = Q_LDS ? 1 : NCH;
-    static_assert(NCH >= 1 && NCH <= kWave && kWave % NCH == 0, "unsupported head dim");
+    static_assert(DH % X == 0 && NCH >= 8 && NCH <= kWave && NCH % CG == 0 && NVL % VG == 0,
+                  "unsupported head dim");
 };
 
 // LDS slot of key k's probability inside a wave's 64-float stage: the V mapping reads, for
-// row group rg = lane/LPR, the NCH consecutive floats [rg*NCH, rg*NCH+NCH) = keys j*RPI+rg.
-template <int NCH, int RPI>
-__device__ __forceinline__ int stage_slot(int k) { return (k % RPI) * NCH + k / RPI; }
+// row group rg = lane/LPR, the NVL consecutive floats [rg*NVL, rg*NVL+NVL) = keys j*RPI+rg.
+template <int NVL, int RPI>
+__device__ __forceinline__ int stage_slot(int k) { return (k % RPI) * NVL + k / RPI; }
 
 // Words exchanged between workgroups of one launch: device-scope relaxed atomics.
 __device__ __forceinline__ void publish(float* p, float v) {
@@ -207,13 +214,12 @@ __device__ __forceinline__ void pv_queue_block(float (&acc)[Elem<T>::X], const S
                                                int count, const char* vc_bh, const char* vnew, int tlen,
                                                int lane) {
     using G = Geo<T, DH>;
-    constexpr int NCH = G::NCH, LPR = G::LPR, RPI = G::RPI;
-    constexpr int VG = NCH < 8 ? NCH : 8;
-    const int rg = lane / LPR, dch = lane % LPR;
-    const float* pw = q.w + block * kWave + rg * NCH;
-    const int* pr = q.row + block * kWave + rg * NCH;
+    constexpr int NCH = G::NCH, LPR = G::LPR, RPI = G::RPI, NVL = G::NVL, VG = G::VG;
+    const int rg = lane / LPR, dch = min(lane % LPR, NCH - 1);
+    const float* pw = q.w + block * kWave + rg * NVL;
+    const int* pr = q.row + block * kWave + rg * NVL;
 #pragma unroll 1
-    for (int g = 0; g < NCH / VG; ++g) {
+    for (int g = 0; g < NVL / VG; ++g) {
         uint4 vv[VG];
         float pj[VG];
 #pragma unroll
@@ -240,7 +246,7 @@ __device__ __forceinline__ void queue_push(float (&acc)[Elem<T>::X], SurvivorQue
         __builtin_amdgcn_mbcnt_hi((unsigned)(mask >> 32), __builtin_amdgcn_mbcnt_lo((unsigned)mask, 0u));
     if (keep) {
         const unsigned n = q.total + before;
-        const int slot = ((n >> 6) & 1) * kWave + stage_slot<G::NCH, G::RPI>(n & 63);
+        const int slot = ((n >> 6) & 1) * kWave + stage_slot<G::NVL, G::RPI>(n & 63);
         q.w[slot] = weight;
         q.row[slot] = key;
     }
@@ -268,7 +274,7 @@ __device__ __forceinline__ void finish_piece(const DecodeParams& P, int bh, int 
                                              float (&acc)[Elem<T>::X], float m_run, float l_run,
                                              float (*s_acc)[DH], float* s_m, float* s_l, int* s_last_p) {
     using G = Geo<T, DH>;
-    constexpr int X = G::X, LPR = G::LPR;
+    constexpr int X = G::X, LPR = G::LPR, NCH = G::NCH;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     int& s_last = *s_last_p;
 #ifdef FFA_TRACE
@@ -285,7 +291,7 @@ __device__ __forceinline__ void finish_piece(const DecodeParams& P, int bh, int 
     // ---- merge the waves of this workgroup (LDS): DH floats + (max, sum) per wave ----
     l_run = wave_sum(l_run);
     if (lane == 0) { s_m[wave] = m_run; s_l[wave] = l_run; }
-    if (lane < LPR) {
+    if (lane < NCH) {
 #pragma unroll
         for (int e = 0; e < X; ++e) s_acc[wave][lane * X + e] = acc[e];
     }
@@ -393,8 +399,8 @@ __device__ __forceinline__ void finish_piece(const DecodeParams& P, int bh, int 
 template <typename T, int DH, int NW>
 __global__ void __launch_bounds__(NW * 64) ffa_decode_split_kernel(const DecodeParams P) {
     using G = Geo<T, DH>;
-    constexpr int X = G::X, NCH = G::NCH, LPR = G::LPR, RPI = G::RPI;
-    constexpr int VG = NCH < 8 ? NCH : 8;  // V loads kept in flight per group
+    constexpr int X = G::X, NCH = G::NCH, LPR = G::LPR, RPI = G::RPI, NVL = G::NVL;
+    constexpr int VG = G::VG;  // V loads kept in flight per group
 
     __shared__ float s_p[NW][kWave];
     __shared__ float s_acc[NW][DH];
@@ -453,7 +459,7 @@ __global__ void __launch_bounds__(NW * 64) ffa_decode_split_kernel(const DecodeP
     NewToken new_tok;
     if (appends) new_tok = new_token_load<NCH>(knew, vnew, lane);
 
-    const int rg = lane / LPR, dch = lane % LPR;
+    const int rg = lane / LPR, dch = min(lane % LPR, NCH - 1);
     float m_run = -INFINITY, l_run = 0.f;
     float acc[X];
 #pragma unroll
@@ -469,7 +475,7 @@ __global__ void __launch_bounds__(NW * 64) ffa_decode_split_kernel(const DecodeP
         }
     };
 
-    constexpr int CG = NCH < 8 ? NCH : 8;
+    constexpr int CG = G::CG;
 
     // First load groups of one tile: CG chunks of K (lane = key) and VG chunks of V
     // (lane = row group x d-chunk).  V does not depend on the scores, so both go out together.
@@ -510,21 +516,21 @@ __global__ void __launch_bounds__(NW * 64) ffa_decode_split_kernel(const DecodeP
         m_run = m_new;
 
         __builtin_amdgcn_wave_barrier();
-        s_p[wave][stage_slot<NCH, RPI>(lane)] = pr;
+        s_p[wave][stage_slot<G::NVL, RPI>(lane)] = pr;
         __builtin_amdgcn_wave_barrier();
 
 #pragma unroll
         for (int e = 0; e < X; ++e) acc[e] *= alpha;
 
         FFA_TP(2);
-        const float* pst = &s_p[wave][rg * NCH];
+        const float* pst = &s_p[wave][rg * NVL];
 #pragma unroll
-        for (int g = 0; g < NCH / VG; ++g) {
+        for (int g = 0; g < NVL / VG; ++g) {
             uint4 vn[VG];
-            if (g + 1 < NCH / VG) load_v_group(vn, tile, g + 1);
+            if (g + 1 < NVL / VG) load_v_group(vn, tile, g + 1);
 #pragma unroll
             for (int j = 0; j < VG; ++j) fma_chunk(acc, pst[g * VG + j], vv[j], T{});
-            if (g + 1 < NCH / VG) {
+            if (g + 1 < NVL / VG) {
 #pragma unroll
                 for (int j = 0; j < VG; ++j) vv[j] = vn[j];
             }
@@ -573,8 +579,7 @@ __global__ void __launch_bounds__(64) ffa_merge_splits_kernel(const DecodeParams
 template <typename T, int DH, int NW>
 __global__ void __launch_bounds__(NW * 64) ffa_decode_wg_kernel(const DecodeParams P) {
     using G = Geo<T, DH>;
-    constexpr int X = G::X, NCH = G::NCH, LPR = G::LPR, RPI = G::RPI;
-    constexpr int VG = NCH < 8 ? NCH : 8;
+    constexpr int X = G::X, NCH = G::NCH, LPR = G::LPR, RPI = G::RPI, NVL = G::NVL, VG = G::VG;
     constexpr int NT = NW * 64;
 
     extern __shared__ float s_dyn[];
@@ -698,7 +703,7 @@ __global__ void __launch_bounds__(NW * 64) ffa_decode_wg_kernel(const DecodePara
     }
 
     // ---- phase 3: P.V.  Pruned: only the surviving rows, compacted per wave ----
-    const int rg = lane / LPR, dch = lane % LPR;
+    const int rg = lane / LPR, dch = min(lane % LPR, NCH - 1);
     float acc[X];
 #pragma unroll
     for (int e = 0; e < X; ++e) acc[e] = 0.f;
@@ -713,7 +718,7 @@ __global__ void __launch_bounds__(NW * 64) ffa_decode_wg_kernel(const DecodePara
     } else {
         for (int tile = tile_lo + wave; tile < ntiles; tile += NW) {
 #pragma unroll 1
-            for (int g = 0; g < NCH / VG; ++g) {
+            for (int g = 0; g < NVL / VG; ++g) {
                 uint4 vv[VG];
                 float pj[VG];
 #pragma unroll
@@ -743,7 +748,7 @@ __global__ void __launch_bounds__(NW * 64) ffa_decode_wg_kernel(const DecodePara
         float o = 0.f;
         for (int w = 0; w < NW; ++w)
 #pragma unroll
-            for (int g = 0; g < RPI; ++g) o += s_acc[w * kWave * X + g * DH + d];
+            for (int g = 0; g < RPI; ++g) o += s_acc[w * kWave * X + g * G::ROWW + d];
         store_out(out, d, all_masked ? 0.f : o * out_scale);
     }
 }
@@ -923,7 +928,7 @@ __global__ void __launch_bounds__(NW * 64) ffa_pruned_pv_kernel(const DecodePara
 #pragma unroll
         for (int e = 0; e < X; ++e) acc[e] += __shfl_xor(acc[e], off);
     }
-    if (lane < LPR) {
+    if (lane < G::NCH) {
 #pragma unroll
         for (int e = 0; e < X; ++e) s_acc[wave][lane * X + e] = acc[e];
     }
@@ -988,8 +993,7 @@ __global__ void __launch_bounds__(256) ffa_init_cache_kernel(uint4* __restrict__
                                                              const uint4* __restrict__ k_src,
                                                              const uint4* __restrict__ v_src,
                                                              int L, int Lmax) {
-    constexpr int PER = TK * NCH / 256;  // chunks per thread, of K and of V
-    static_assert(TK * NCH % 256 == 0 && PER >= 1, "tile must divide over the workgroup");
+    constexpr int PER = (TK * NCH + 255) / 256;  // chunks per thread, of K and of V
     __shared__ uint4 s_tile[NCH * (TK + 1)];  // [chunk][key], one chunk of padding per row
     const int bh = blockIdx.y;
     const int l0 = blockIdx.x * TK;
@@ -1009,15 +1013,15 @@ __global__ void __launch_bounds__(256) ffa_init_cache_kernel(uint4* __restrict__
 #pragma unroll
     for (int j = 0; j < PER; ++j) {
         const int i = threadIdx.x + j * 256;
-        if (i < n) vd[i] = vv[j];                              // V: contiguous copy
-        s_tile[(i % NCH) * (TK + 1) + i / NCH] = kv[j];        // K: [key][chunk] -> [chunk][key]
+        if (i < n) vd[i] = vv[j];                                            // V: contiguous copy
+        if (i < TK * NCH) s_tile[(i % NCH) * (TK + 1) + i / NCH] = kv[j];   // K: [key][chunk] -> [chunk][key]
     }
     __syncthreads();
 #pragma unroll
     for (int j = 0; j < PER; ++j) {
         const int i = threadIdx.x + j * 256;
         const int c = i / TK, key = i % TK;
-        if (key * NCH < n) kd[(size_t)c * Lmax + key] = s_tile[c * (TK + 1) + key];
+        if (c < NCH && key * NCH < n) kd[(size_t)c * Lmax + key] = s_tile[c * (TK + 1) + key];
     }
 }
 
@@ -1106,6 +1110,7 @@ static int dispatch_head_dim(const DecodeParams& P, int head_dim, const ffa_laun
                              hipStream_t st) {
     switch (head_dim) {
         case 64: return dispatch_waves<T, 64>(P, plan, st);
+        case 80: return dispatch_waves<T, 80>(P, plan, st);
         case 128: return dispatch_waves<T, 128>(P, plan, st);
         case 256: return dispatch_waves<T, 256>(P, plan, st);
         default: return FFA_ERR_HEAD_DIM;
@@ -1144,13 +1149,13 @@ int launch_decode(const DecodeArgs& a, const ffa_launch_plan& plan, const Worksp
 int launch_init_cache(int precision, void* k_dst, void* v_dst, const void* k_src,
                       const void* v_src, int B, int H, int L, int Lmax, int Dh, void* stream) {
     const int nch = Dh * (precision / 8) / 16;
-    if (nch != 8 && nch != 16 && nch != 32 && nch != 64) return FFA_ERR_HEAD_DIM;
+    if (nch != 8 && nch != 10 && nch != 16 && nch != 20 && nch != 32 && nch != 64) return FFA_ERR_HEAD_DIM;
     if (L <= 0) return FFA_OK;
     // 512 chunks (8 KiB of K, 8 KiB of V) per workgroup: measured against 1024 / 2048 / 4096,
     // the small tile wins at every shape -- many resident workgroups hide the latency better
     // than more loads per thread do.
     constexpr int kIc = 512;
-    const int tk = kIc / nch;
+    const int tk = nch == 10 ? 64 : nch == 20 ? 32 : kIc / nch;  // Dh = 80: 640 chunks
     const dim3 grid((unsigned)((L + tk - 1) / tk), (unsigned)(B * H));
     hipStream_t st = reinterpret_cast<hipStream_t>(stream);
     auto kd = reinterpret_cast<uint4*>(k_dst);
@@ -1162,6 +1167,8 @@ int launch_init_cache(int precision, void* k_dst, void* v_dst, const void* k_src
         case 16: hipLaunchKernelGGL((ffa_init_cache_kernel<16, kIc / 16>), grid, dim3(256), 0, st, kd, vd, ks, vs, L, Lmax); break;
         case 32: hipLaunchKernelGGL((ffa_init_cache_kernel<32, kIc / 32>), grid, dim3(256), 0, st, kd, vd, ks, vs, L, Lmax); break;
         case 64: hipLaunchKernelGGL((ffa_init_cache_kernel<64, kIc / 64>), grid, dim3(256), 0, st, kd, vd, ks, vs, L, Lmax); break;
+        case 10: hipLaunchKernelGGL((ffa_init_cache_kernel<10, 64>), grid, dim3(256), 0, st, kd, vd, ks, vs, L, Lmax); break;
+        case 20: hipLaunchKernelGGL((ffa_init_cache_kernel<20, 32>), grid, dim3(256), 0, st, kd, vd, ks, vs, L, Lmax); break;
         default: return FFA_ERR_HEAD_DIM;
     }
     return check_launch();

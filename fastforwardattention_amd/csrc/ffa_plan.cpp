@@ -44,7 +44,7 @@ int plan_launch(int precision, int B, int H, int Dh, int t, float p, int use_def
                 ffa_launch_plan* plan) {
     if (plan == nullptr) return FFA_ERR_NULL_POINTER;
     if (precision != FFA_PRECISION_F16 && precision != FFA_PRECISION_F32) return FFA_ERR_DTYPE;
-    if (Dh != 64 && Dh != 128 && Dh != 256) return FFA_ERR_HEAD_DIM;
+    if (Dh != 64 && Dh != 80 && Dh != 128 && Dh != 256) return FFA_ERR_HEAD_DIM;
     if (B <= 0 || H <= 0) return FFA_ERR_SHAPE;
     if (t < 0) return FFA_ERR_TIMESTEP;
     if (!(p >= 0.f)) return FFA_ERR_PROB_THRESH;

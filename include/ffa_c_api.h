@@ -36,7 +36,7 @@ typedef enum ffa_status {
     FFA_OK = 0,
     FFA_ERR_NULL_POINTER = 1,   /* a required pointer is NULL                                */
     FFA_ERR_DTYPE = 2,          /* precision is neither 16 nor 32                            */
-    FFA_ERR_HEAD_DIM = 3,       /* Dh not one of 64, 128, 256                                */
+    FFA_ERR_HEAD_DIM = 3,       /* Dh not one of 64, 80, 128, 256                            */
     FFA_ERR_SHAPE = 4,          /* B, H, L or Lmax not positive, or L > Lmax                 */
     FFA_ERR_TIMESTEP = 5,       /* t outside [0, Lmax)                                       */
     FFA_ERR_ALIGNMENT = 6,      /* a pointer is not 16-byte aligned                          */

@@ -87,7 +87,7 @@ def test_errors_raise():
     with pytest.raises(RuntimeError, match="prob_thresh"):
         ffa.attention(q, q, q, 0.1, 10, -1.0)
     with pytest.raises(RuntimeError, match="head dim"):
-        FFA(torch.randn(1, 2, 10, 80).half().cuda(), torch.randn(1, 2, 10, 80).half().cuda(), 12, False)
+        FFA(torch.randn(1, 2, 10, 96).half().cuda(), torch.randn(1, 2, 10, 96).half().cuda(), 12, False)
     with pytest.raises(RuntimeError):
         FFA(torch.randn(1, 2, 10, 64).double().cuda(), torch.randn(1, 2, 10, 64).double().cuda(), 12, False)
     with pytest.raises(TypeError):

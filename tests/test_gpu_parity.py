@@ -60,7 +60,7 @@ def _plans(prec, B, H, Dh, t):
 
 # ------------------------------------------------------------------ cache construction
 @pytest.mark.parametrize("prec", [16, 32])
-@pytest.mark.parametrize("Dh", [64, 128, 256])
+@pytest.mark.parametrize("Dh", [64, 80, 128, 256])
 @pytest.mark.parametrize("L,Lmax", [(1, 1), (63, 64), (64, 80), (130, 131), (257, 400)])
 def test_init_cache_bit_exact(prec, Dh, L, Lmax):
     _say("init_cache", prec, Dh, L, Lmax)
@@ -76,7 +76,7 @@ def test_init_cache_bit_exact(prec, Dh, L, Lmax):
 
 # ------------------------------------------------------------------ exact decode, one step
 @pytest.mark.parametrize("prec", [16, 32])
-@pytest.mark.parametrize("Dh", [64, 128, 256])
+@pytest.mark.parametrize("Dh", [64, 80, 128, 256])
 @pytest.mark.parametrize("t", [0, 1, 63, 64, 65, 200, 777])
 def test_exact_step_all_plans(prec, Dh, t):
     B, H = 2, 3
@@ -119,7 +119,8 @@ def test_known_answers():
 
 # ------------------------------------------------------------------ iterative decode
 @pytest.mark.parametrize("prec,Dh,B,H,L,steps", [(16, 64, 2, 32, 1000, 24), (32, 64, 1, 8, 120, 20),
-                                                 (16, 256, 2, 4, 500, 12), (16, 128, 1, 5, 61, 10)])
+                                                 (16, 256, 2, 4, 500, 12), (16, 128, 1, 5, 61, 10),
+                                                 (16, 80, 2, 32, 300, 12), (32, 80, 1, 3, 130, 8)])
 @pytest.mark.parametrize("use_default", [False, True])
 def test_iterative_decode_every_step(prec, Dh, B, H, L, steps, use_default):
     """BASELINE config 2 in miniature: prompt cache, then `steps` appended tokens, parity at
@@ -234,7 +235,7 @@ def _near_threshold(prec, P, thr):
 
 
 @pytest.mark.parametrize("prec", [16, 32])
-@pytest.mark.parametrize("Dh,L", [(64, 900), (256, 300)])
+@pytest.mark.parametrize("Dh,L", [(64, 900), (80, 500), (256, 300)])
 @pytest.mark.parametrize("p", [1e-4, 1e-3, 1e-2, 0.3])
 def test_pruned_step_matches_rule(prec, Dh, L, p):
     """Skip set and output against the CPU transcription of attention.cu's pruning rule.

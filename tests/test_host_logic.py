@@ -62,7 +62,7 @@ def _attn(lib, precision=16, B=2, H=4, Dh=64, Lmax=128, scale=0.125, t=10, q=P, 
 def test_attention_argument_validation(lib):
     wg = capi.make_plan(capi.FFA_LAUNCH_WORKGROUP, 4, 1, 1)
     assert _attn(lib, precision=8, plan=wg) == 2          # dtype
-    assert _attn(lib, Dh=80, plan=wg) == 3                # head dim (80 is a reference size we do not ship)
+    assert _attn(lib, Dh=96, plan=wg) == 3                # head dim: 64, 80, 128, 256 like the reference
     assert _attn(lib, B=0, plan=wg) == 4
     assert _attn(lib, H=-1, plan=wg) == 4
     assert _attn(lib, t=-1, plan=wg) == 5
@@ -129,7 +129,7 @@ def test_workspace_bytes_covers_every_plan(lib):
 
 
 @pytest.mark.parametrize("prec", [16, 32])
-@pytest.mark.parametrize("Dh", [64, 128, 256])
+@pytest.mark.parametrize("Dh", [64, 80, 128, 256])
 def test_planner_consistency(prec, Dh):
     for B, H in [(1, 1), (1, 32), (2, 32), (10, 32), (16, 32), (64, 64)]:
         for t in [0, 1, 31, 63, 64, 127, 999, 1000, 1255, 2047, 2048, 8191, 16383, 30000]:
@@ -175,7 +175,8 @@ def test_planner_rejects_bad_input(lib):
     plan = capi.LaunchPlan()
     f = lib.ffa_plan_launch
     assert f(8, 1, 1, 64, 10, 0.0, 0, 256, C.byref(plan)) == 2
-    assert f(16, 1, 1, 80, 10, 0.0, 0, 256, C.byref(plan)) == 3
+    assert f(16, 1, 1, 96, 10, 0.0, 0, 256, C.byref(plan)) == 3
+    assert f(16, 1, 1, 80, 10, 0.0, 0, 256, C.byref(plan)) == 0
     assert f(16, 0, 1, 64, 10, 0.0, 0, 256, C.byref(plan)) == 4
     assert f(16, 1, 1, 64, -1, 0.0, 0, 256, C.byref(plan)) == 5
     assert f(16, 1, 1, 64, 10, -1.0, 0, 256, C.byref(plan)) == 10
