@@ -100,6 +100,15 @@ int plan_launch(int precision, int B, int H, int Dh, int t, float p, int use_def
     //    cover all CUs and are done, merges included, long before the whole pairs are.
     //  - Fewer pairs than CUs: floor(CUs/pairs) pieces per pair (one workgroup per CU), but
     //    never so many that a wave is left without a tile.
+    //  - Long sequences with at least one pair per CU: the one-workgroup kernel with 16 waves
+    //    (70 VGPRs, two workgroups = 32 waves resident per CU, separate K and V phases) streams
+    //    3-6 % faster than the split kernel (8192 keys: 256 pairs 104 vs 111 us, 512 pairs
+    //    205 vs 214 us, 1024 pairs 395 vs 412 us; 4096 keys: 95 vs 98, 184 vs 191 us); below
+    //    4096 keys the split kernel is ahead.
+    if (bh >= cus && ntiles >= 64 && fits_wg) {
+        fill(plan, FFA_LAUNCH_WORKGROUP, 16, 1, ntiles);
+        return FFA_OK;
+    }
     const int waves = wg_waves_for(ntiles, 4);
     int whole = (bh / cus) * cus;
     const int rest = bh - whole;

@@ -153,6 +153,9 @@ def test_planner_consistency(prec, Dh):
                             assert (plan.n_splits - 1) * plan.tiles_per_split < ntiles  # no empty piece
                             assert B * H * plan.n_splits <= max(512, B * H)              # about two per CU
                             assert plan.waves_per_wg <= 8 and plan.whole_heads == 0
+                    elif B * H >= 256 and ntiles >= 64 and fits_lds:
+                        # many pairs, long sequence: the 16-wave one-workgroup kernel streams best
+                        assert plan.kind == capi.FFA_LAUNCH_WORKGROUP and plan.waves_per_wg == 16
                     else:
                         assert plan.kind == capi.FFA_LAUNCH_SPLIT
                         assert (plan.n_splits - 1) * plan.tiles_per_split < ntiles  # no empty split
