@@ -514,7 +514,7 @@ def main():
         "ms_per_step": round(us_step / 1e3, 6), "us_per_step": round(us_step, 3),
         "tokens_per_s": round(wl.B / (us_step * 1e-6), 1),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "f16 (fp32 accumulate)", "data": "synthetic",
+        "dtype": "f16", "accumulate_dtype": "f32", "data": "synthetic",
         "config": {"workload": f"{args.workload}: B={wl.B} H={wl.H} Dh={wl.Dh} fp16 prompt={wl.prompt} "
                                f"t={wl.prompt}->{wl.prompt + min(wl.gen, -(-steps // wl.layers))} p=0 "
                                f"scale={wl.scale}; step = one attention call on one of {wl.layers} "
