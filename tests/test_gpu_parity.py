@@ -343,3 +343,79 @@ def test_full_size_config2_properties():
     sess1 = CApiSession(K.numpy(), ones, Lmax)
     c = sess1.step(q.numpy(), k.numpy(), np.ones((B, H, Dh), np.float16), 0.125, L)
     np.testing.assert_allclose(c, 1.0, atol=1e-3)
+
+
+# ------------------------------------------------------------------ randomized sweep
+def _random_plan(rng, prec, B, H, Dh, t, p):
+    ntiles = t // 64 + 1
+    kinds = ["library", "default", "workgroup", "two_pass"] + (["split"] * 2 if p == 0 else [])
+    kind = kinds[rng.integers(len(kinds))]
+    if kind == "library":
+        return kind, None
+    if kind == "default":
+        return kind, capi.plan_launch(prec, B, H, Dh, t, p, True)
+    if kind == "workgroup":
+        return kind, capi.make_plan(capi.FFA_LAUNCH_WORKGROUP, int(rng.choice([1, 2, 4, 8, 16])), 1, ntiles)
+    waves = int(rng.choice([1, 2, 4, 8]))
+    tps = int(rng.integers(1, ntiles + 1))
+    ns = -(-ntiles // tps)
+    if ns > 128:
+        tps, ns = ntiles, 1
+    if kind == "two_pass":
+        return kind, capi.make_plan(capi.FFA_LAUNCH_TWO_PASS, waves, ns, tps)
+    whole = int(rng.integers(0, B * H + 1))
+    combine = int(rng.integers(2))
+    return kind, capi.make_plan(capi.FFA_LAUNCH_SPLIT, waves, ns, tps, combine, whole)
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_random_shapes_plans_and_padding(seed):
+    """Random head dims, lengths, paddings, thresholds and launch plans (every kind, every wave
+    count, ragged pieces), ten cases per seed, each against the oracle."""
+    rng = np.random.default_rng(1000 + seed)
+    for case in range(10):
+        prec = int(rng.choice([16, 32]))
+        Dh = int(rng.choice([64, 80, 128, 256]))
+        B, H = int(rng.integers(1, 4)), int(rng.integers(1, 6))
+        t = int(rng.choice([0, 1, 63, 64, 65, 127, 128, int(rng.integers(2, 700))]))
+        Lmax = t + int(rng.integers(1, 70))
+        p = float(rng.choice([0.0, 0.0, 1e-3, 0.05]))
+        pad = str(rng.choice(["none", "left", "right"]))
+        K, V, q, k, v = _peaked(prec, int(rng.integers(1 << 30)), B, H, t, Dh, npeaks=min(8, t))
+        scale = 1.0 / np.sqrt(Dh)
+        sl, rnp = None, True
+        if pad == "left":
+            sl, rnp = rng.integers(0, t + 2, B).astype(np.int32), False      # t+1: every key masked
+        elif pad == "right":
+            sl = rng.integers(0, t + 1, B).astype(np.int32)
+        kind, plan = _random_plan(rng, prec, B, H, Dh, t, p)
+        _say("random", seed, case, dict(prec=prec, Dh=Dh, B=B, H=H, t=t, Lmax=Lmax, p=p, pad=pad,
+                                        sl=None if sl is None else sl.tolist(), kind=kind, plan=plan))
+        kc0, vc0 = O.pack_k_cache(K, Lmax), O.pack_v_cache(V, Lmax)
+        sess = CApiSession(K, V, Lmax)
+        if p == 0.0:
+            want = O.decode_step(q, k, v, kc0, vc0, scale, t, seq_lengths=sl, right_or_no_padding=rnp,
+                                 acc=np.float64)
+            got = sess.step(q, k, v, scale, t, plan=plan, seq_lengths=sl, right_or_no_padding=rnp)
+            assert float(np.abs(got - want).max()) <= _tol(prec, V, v)
+        else:
+            want, skip, P, thr = O.pruned_decode_step(q, k, v, kc0, vc0, scale, t, p, seq_lengths=sl,
+                                                      right_or_no_padding=rnp)
+            got, kept, gmask = sess.step(q, k, v, scale, t, p=p, plan=plan, seq_lengths=sl,
+                                         right_or_no_padding=rnp, diag=True)
+            diff = gmask != skip
+            assert not (diff & ~_near_threshold(prec, P, thr)).any()
+            tl = np.full(B, t) if (sl is None or not rnp) else sl
+            for b in range(B):
+                n = int(tl[b])
+                np.testing.assert_array_equal(kept[b], n - gmask[b, :, :n].sum(axis=-1))
+                Vb = np.concatenate([V[b, :, :n], v[b, :, None]], axis=1).astype(np.float32)
+                w = np.where(gmask[b, :, :n + 1], 0, P[b, :, :n + 1])
+                want_g = np.einsum("hn,hnd->hd", w, Vb)
+                assert float(np.abs(got[b] - want_g).max()) <= (1e-3 if prec == 16 else 1e-5) * max(1.0, float(np.abs(Vb).max()))
+        gk, gv = sess.caches()
+        tl = np.full(B, t) if (sl is None or not rnp) else sl
+        for b in range(B):        # caches: prompt + the appended token, bit for bit
+            n = int(tl[b]) + 1
+            np.testing.assert_array_equal(gk[b, :, :, :n], kc0[b, :, :, :n])
+            np.testing.assert_array_equal(gv[b, :, :n], vc0[b, :, :n])
