@@ -198,6 +198,40 @@ def run_ext(wl, steps, warmup):
     return time_region(torch, body)
 
 
+def parity_check(wl):
+    """The workload's whole decode loop on one layer cache, untimed: fp16 kernel output through
+    the C ABI (the library's own launch plan at every step) against fp32 torch on the GPU
+    (softmax(q K^T scale) V over the upcast fp16 inputs).  Returns the worst max-abs error."""
+    torch, capi, lib = wl.torch, wl.capi, wl.lib
+    B, H, Dh, L, Lmax, gen = wl.B, wl.H, wl.Dh, wl.prompt, wl.Lmax, wl.gen
+    dev = "cuda:0"
+    g = torch.Generator(device=dev).manual_seed(1)
+    K = (torch.randn(B, H, L, Dh, device=dev, generator=g) * 0.5).half()
+    V = (torch.randn(B, H, L, Dh, device=dev, generator=g) * 0.5).half()
+    kc = torch.empty(B, H, Dh // 8, Lmax, 8, dtype=torch.float16, device=dev)
+    vc = torch.empty(B, H, Lmax, Dh, dtype=torch.float16, device=dev)
+    capi.check(lib.ffa_init_cache_f16(kc.data_ptr(), vc.data_ptr(), K.data_ptr(), V.data_ptr(),
+                                      B, L, Lmax, Dh, H, None), "ffa_init_cache_f16")
+    Kf = torch.zeros(B * H, Lmax, Dh, device=dev)
+    Vf = torch.zeros(B * H, Lmax, Dh, device=dev)
+    Kf[:, :L], Vf[:, :L] = K.float().reshape(B * H, L, Dh), V.float().reshape(B * H, L, Dh)
+    out = torch.empty(B, H, Dh, dtype=torch.float16, device=dev)
+    worst = 0.0
+    for i in range(gen):
+        t = L + i
+        q, k, v = (torch.randn(B, H, Dh, device=dev, generator=g).half() for _ in range(3))
+        plan = wl.plan_for(t)
+        capi.check(lib.ffa_attention_f16(B, H, Dh, Lmax, wl.scale, t, q.data_ptr(), k.data_ptr(), v.data_ptr(),
+                                         kc.data_ptr(), vc.data_ptr(), out.data_ptr(), None, 0.0, C.byref(plan), 1,
+                                         wl.ws.data_ptr(), wl.ws_bytes, None), "ffa_attention_f16")
+        Kf[:, t], Vf[:, t] = k.float().reshape(B * H, Dh), v.float().reshape(B * H, Dh)
+        w = torch.softmax(torch.bmm(q.float().reshape(B * H, 1, Dh), Kf[:, :t + 1].transpose(1, 2)) * wl.scale, -1)
+        ref = torch.bmm(w, Vf[:, :t + 1]).reshape(B, H, Dh)
+        worst = max(worst, float((out.float() - ref).abs().max()))
+    return {"max_abs_err": worst, "tolerance": 1e-3, "steps": gen, "ok": worst <= 1e-3,
+            "reference": "fp32 torch bmm/softmax/bmm on the GPU over the upcast fp16 inputs, every step"}
+
+
 def cpu_baseline(wl, budget_s=15.0, max_steps=64):
     """The reference's CPU path restated (oracle/torch_attn.py) on the host cores, on the
     first steps of the same workload (one layer's cache), bounded by a time budget."""
@@ -456,6 +490,7 @@ def main():
     ap.add_argument("--plan", default=None, help="kind,waves,tiles_per_split[,combine[,whole_heads]] (kind: 0 workgroup, 1 split; combine: 0 fused, 1 kernel)")
     ap.add_argument("--legs", default="graph,capi,ext", help="comma list of graph,capi,ext")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-parity", action="store_true", help="skip the untimed every-step parity check")
     ap.add_argument("--suite", action="store_true",
                     help="run every BASELINE configuration (tuned and default launch) and the pruned sweep; "
                          "one JSON line each instead of the single headline line")
@@ -533,9 +568,14 @@ def main():
             u = res[leg] * 1e3 / steps
             out[f"eager_{leg}_us_per_step"] = round(u, 3)
             out[f"eager_{leg}_GBps"] = round(mean_b / (u * 1e-6) / 1e9, 1)
+    if not args.no_parity:
+        out["parity"] = parity_check(wl)
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(wl)
     print(json.dumps(out))
+    if not args.no_parity and not out["parity"]["ok"]:
+        print("bench.py: parity check FAILED; the throughput above is not a valid result", file=sys.stderr)
+        sys.exit(4)
 
 
 if __name__ == "__main__":
