@@ -125,6 +125,13 @@ int plan_launch(int precision, int B, int H, int Dh, int t, float p, int use_def
     const int tps = ceil_div(ntiles, n_splits);
     n_splits = ceil_div(ntiles, tps);
     if (n_splits == 1) whole = bh;  // nothing left to split: plain one-workgroup-per-pair
+    // Between CUs/2 and CUs pairs nothing can be cut without doubling up CUs; the idle CUs
+    // are made up for with 8 waves per workgroup (160 pairs, 1000 keys: 9.8 vs 10.1 us).
+    if (n_splits == 1 && bh < cus) {
+        fill(plan, FFA_LAUNCH_SPLIT, wg_waves_for(ntiles, 8), 1, ntiles);
+        plan->whole_heads = bh;
+        return FFA_OK;
+    }
     fill(plan, FFA_LAUNCH_SPLIT, waves, n_splits, tps);
     plan->whole_heads = whole;
     return FFA_OK;
