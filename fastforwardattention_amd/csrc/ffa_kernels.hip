@@ -195,6 +195,10 @@ __device__ __forceinline__ void publish(float* p, float v) {
 __device__ __forceinline__ float acquire(const float* p) {
     return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
+// Waits until this lane's outstanding vector memory operations, published stores included,
+// have been acknowledged.  A workgroup barrier alone does not: it orders the waves of one CU,
+// not their stores on the way to memory.
+__device__ __forceinline__ void wait_published() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
 
 // ---------------------------------------------------------------------------------------
 // Survivor queue of the pruning kernels.  A key that the rule drops must cost neither bytes
@@ -335,9 +339,9 @@ __device__ __forceinline__ void finish_piece(const DecodeParams& P, int bh, int 
     // No device-scope fence here: on this part such a fence writes back / invalidates a
     // whole L2 and costs far more than the kernel itself.  Instead every word that crosses
     // workgroups is moved with device-scope atomic accesses, which the hardware performs
-    // at the level all XCDs share, so nothing needs flushing.  Order: each thread's
-    // published stores are complete before the workgroup barrier (the barrier waits for
-    // outstanding memory operations), the arrival counter is bumped after it, and the
+    // at the level all XCDs share, so nothing needs flushing.  Order: every thread waits
+    // until its own published stores have been acknowledged (wait_published) and only then
+    // enters the workgroup barrier; the arrival counter is bumped after the barrier, and the
     // merging workgroup reads the partials only after it has seen the final count.
     if (tid == 0) {
         float* ml = P.ws_ml + (slot0 + split) * 2;
@@ -345,6 +349,7 @@ __device__ __forceinline__ void finish_piece(const DecodeParams& P, int bh, int 
         publish(&ml[1], L);
     }
     FFA_TP(4);
+    wait_published();
     __syncthreads();
     FFA_TP(5);
     if (tid == 0) {
@@ -953,8 +958,9 @@ __global__ void __launch_bounds__(NW * 64) ffa_pruned_pv_kernel(const DecodePara
     }
     if (P.n_splits == 1) return;
 
-    // Same publication protocol as ffa_decode_split_kernel (device-scope relaxed atomics,
-    // ordered by the workgroup barrier and the arrival counter; no fences).
+    // Same publication protocol as ffa_decode_split_kernel (device-scope relaxed atomics;
+    // stores acknowledged, then the workgroup barrier, then the arrival counter; no fences).
+    wait_published();
     __syncthreads();
     if (tid == 0) {
         const unsigned prev =
