@@ -419,3 +419,44 @@ def test_random_shapes_plans_and_padding(seed):
             n = int(tl[b]) + 1
             np.testing.assert_array_equal(gk[b, :, :, :n], kc0[b, :, :, :n])
             np.testing.assert_array_equal(gv[b, :, :n], vc0[b, :, :n])
+
+
+@pytest.mark.parametrize("prec,iters", [(16, 300), (32, 1200)])
+def test_cross_workgroup_merge_stress(prec, iters):
+    """Many launches of the hybrid whole/split plan (the pieces publish their partials while
+    the whole pairs still stream at full bandwidth) and of a merge-heavy plan, against the
+    one-workgroup kernel on the same inputs: a partial that is read before it has arrived
+    shows up as a large error in some pair of some launch."""
+    B, H, Dh, t = 10, 32, 64, 1100
+    rng, K, V = rand_inputs(21, B, H, t, Dh, prec)
+    Lmax = t + 4
+    sess = CApiSession(K, V, Lmax)
+    ntiles = t // 64 + 1
+    wg = capi.make_plan(capi.FFA_LAUNCH_WORKGROUP, 8, 1, ntiles)
+    hybrid = capi.make_plan(capi.FFA_LAUNCH_SPLIT, 4, -(-ntiles // 5), 5, 0, 256)
+    fine = capi.make_plan(capi.FFA_LAUNCH_SPLIT, 4, -(-ntiles // 2), 2, 0, 0)
+    two_pass = capi.make_plan(capi.FFA_LAUNCH_TWO_PASS, 4, -(-ntiles // 2), 2)
+    tol = 1e-3 if prec == 16 else 2e-6
+    dev, tdt = "cuda:0", torch.float16 if prec == 16 else torch.float32
+    out = torch.empty(B, H, Dh, dtype=tdt, device=dev)
+    ref = torch.empty(B, H, Dh, dtype=tdt, device=dev)
+    fn = sess.lib.ffa_attention_f16 if prec == 16 else sess.lib.ffa_attention_f32
+    from tests.ffa_testlib import ptr
+    import ctypes as C
+
+    def launch(plan, q, k, v, dst):
+        rc = fn(B, H, Dh, Lmax, 0.125, t, ptr(q), ptr(k), ptr(v), ptr(sess.k_cache), ptr(sess.v_cache), ptr(dst),
+                None, 0.0, C.byref(plan), 1, ptr(sess.ws), sess.ws.numel(), None)
+        assert rc == 0
+
+    g = torch.Generator(device=dev).manual_seed(3)
+    worst = 0.0
+    for it in range(iters):
+        q, k, v = (torch.randn(B, H, Dh, device=dev, generator=g).to(tdt) for _ in range(3))
+        launch(wg, q, k, v, ref)
+        for plan in (hybrid, fine, two_pass) if it % 4 == 0 else (hybrid,):
+            launch(plan, q, k, v, out)
+            err = float((out.float() - ref.float()).abs().max())
+            worst = max(worst, err)
+            assert err <= tol, (it, plan, err)
+    _say("merge stress", prec, iters, "launches, worst difference", worst)
