@@ -87,6 +87,16 @@ def test_attention_argument_validation(lib):
     sp = capi.make_plan(capi.FFA_LAUNCH_SPLIT, 4, 2, 1)
     assert _attn(lib, t=100, plan=sp) == 7
     assert _attn(lib, t=100, plan=sp, ws=P, ws_bytes=64) == 7
+    # two-pass plans: coverage, wave count, whole_heads, workspace
+    tp = capi.make_plan(capi.FFA_LAUNCH_TWO_PASS, 4, 2, 1)
+    assert _attn(lib, t=100, plan=tp) == 7
+    assert _attn(lib, t=100, plan=tp, ws=P, ws_bytes=4096) == 7                      # scores do not fit
+    assert _attn(lib, t=200, Lmax=256, plan=tp, ws=P, ws_bytes=1 << 20) == 8         # 2 tiles < 4 needed
+    assert _attn(lib, t=100, plan=capi.make_plan(capi.FFA_LAUNCH_TWO_PASS, 16, 2, 1), ws=P, ws_bytes=1 << 20) == 8
+    assert _attn(lib, t=100, plan=capi.make_plan(capi.FFA_LAUNCH_TWO_PASS, 4, 2, 1, whole_heads=1), ws=P,
+                 ws_bytes=1 << 20) == 8
+    assert _attn(lib, t=100, plan=capi.make_plan(capi.FFA_LAUNCH_TWO_PASS, 4, 2, 1, combine=1), ws=P,
+                 ws_bytes=1 << 20) == 8
     # one-workgroup launch whose scores cannot fit in LDS
     assert _attn(lib, t=60000, Lmax=65536, plan=wg) == 9
 
