@@ -43,6 +43,7 @@ WORKLOADS = {
     "opt1.3b_b5": dict(B=5, H=32, Dh=64, prompt=1000, gen=256, scale=0.125, layers=24),
     "opt1.3b_b2": dict(B=2, H=32, Dh=64, prompt=1000, gen=256, scale=0.125, layers=24),
     "opt1.3b_b1": dict(B=1, H=32, Dh=64, prompt=1000, gen=256, scale=0.125, layers=24),
+    "opt1.3b_b10_f32": dict(B=10, H=32, Dh=64, prompt=1000, gen=256, scale=0.125, layers=24, dtype="f32"),
     "opt2.7b_b10": dict(B=10, H=32, Dh=80, prompt=1000, gen=256, scale=80 ** -0.5, layers=32),
     "gptj_b8": dict(B=8, H=16, Dh=256, prompt=2000, gen=256, scale=0.0625, layers=8),
     "long_b1_16k": dict(B=1, H=32, Dh=64, prompt=16384 - 128, gen=128, scale=0.125, layers=24),
@@ -71,27 +72,34 @@ class Workload:
         self.Lmax = self.prompt + self.gen
         self.use_default = use_default
         self.plan_override = plan_override
+        self.dtype = w.get("dtype", "f16")
+        self.elem = 2 if self.dtype == "f16" else 4
+        self.precision = 8 * self.elem
+        self.tdtype = torch.float16 if self.dtype == "f16" else torch.float32
+        self.fn_init = self.lib.ffa_init_cache_f16 if self.dtype == "f16" else self.lib.ffa_init_cache_f32
+        self.fn_attn = self.lib.ffa_attention_f16 if self.dtype == "f16" else self.lib.ffa_attention_f32
+        x, tdt = 16 // self.elem, self.tdtype
         dev = "cuda:0"
         B, H, Dh, L, Lmax = self.B, self.H, self.Dh, self.prompt, self.Lmax
         g = torch.Generator(device=dev).manual_seed(0)
         self.kc, self.vc = [], []
         for _ in range(self.layers):
-            K = (torch.randn(B, H, L, Dh, device=dev, generator=g) * 0.5).half()
-            V = (torch.randn(B, H, L, Dh, device=dev, generator=g) * 0.5).half()
-            kc = torch.empty(B, H, Dh // 8, Lmax, 8, dtype=torch.float16, device=dev)
-            vc = torch.empty(B, H, Lmax, Dh, dtype=torch.float16, device=dev)
-            capi.check(self.lib.ffa_init_cache_f16(kc.data_ptr(), vc.data_ptr(), K.data_ptr(), V.data_ptr(),
-                                                   B, L, Lmax, Dh, H, None), "ffa_init_cache_f16")
+            K = (torch.randn(B, H, L, Dh, device=dev, generator=g) * 0.5).to(tdt)
+            V = (torch.randn(B, H, L, Dh, device=dev, generator=g) * 0.5).to(tdt)
+            kc = torch.empty(B, H, Dh // x, Lmax, x, dtype=tdt, device=dev)
+            vc = torch.empty(B, H, Lmax, Dh, dtype=tdt, device=dev)
+            capi.check(self.fn_init(kc.data_ptr(), vc.data_ptr(), K.data_ptr(), V.data_ptr(),
+                                    B, L, Lmax, Dh, H, None), "ffa_init_cache")
             torch.cuda.synchronize()
             self.kc.append(kc)
             self.vc.append(vc)
             del K, V
         # a ring of fresh q/k/v tokens (N(0,1)), resident in HBM before the timed region
         self.ring = 64
-        self.q = torch.randn(self.ring, B, H, Dh, device=dev, generator=g).half()
-        self.k = torch.randn(self.ring, B, H, Dh, device=dev, generator=g).half()
-        self.v = torch.randn(self.ring, B, H, Dh, device=dev, generator=g).half()
-        self.out = torch.empty(self.ring, B, H, Dh, dtype=torch.float16, device=dev)
+        self.q = torch.randn(self.ring, B, H, Dh, device=dev, generator=g).to(tdt)
+        self.k = torch.randn(self.ring, B, H, Dh, device=dev, generator=g).to(tdt)
+        self.v = torch.randn(self.ring, B, H, Dh, device=dev, generator=g).to(tdt)
+        self.out = torch.empty(self.ring, B, H, Dh, dtype=tdt, device=dev)
         nbytes = self.lib.ffa_workspace_bytes(B, H, Dh, Lmax)
         self.ws = torch.zeros(nbytes, dtype=torch.uint8, device=dev)
         self.ws_bytes = nbytes
@@ -113,7 +121,7 @@ class Workload:
                 p = self.capi.make_plan(kind, waves, ns, ntiles if ns == 1 and kind == 0 else tps, combine,
                                         whole)
             else:
-                p = self.capi.plan_launch(16, self.B, self.H, self.Dh, t, 0.0, self.use_default,
+                p = self.capi.plan_launch(self.precision, self.B, self.H, self.Dh, t, 0.0, self.use_default,
                                           self.lib.ffa_device_compute_units())
             self._plans[t] = p
         return p
@@ -122,16 +130,16 @@ class Workload:
         """One step through the C ABI (no allocation, no sync)."""
         t = self.t_of(i)
         r, l = i % self.ring, i % self.layers
-        rc = self.lib.ffa_attention_f16(
+        rc = self.fn_attn(
             self.B, self.H, self.Dh, self.Lmax, self.scale, t,
             self.q[r].data_ptr(), self.k[r].data_ptr(), self.v[r].data_ptr(),
             self.kc[l].data_ptr(), self.vc[l].data_ptr(), self.out[r].data_ptr(), None, 0.0,
             C.byref(self.plan_for(t)), 1, self.ws.data_ptr(), self.ws_bytes, stream_ptr)
         if rc != 0:
-            raise RuntimeError(f"ffa_attention_f16 failed: {self.capi.status_string(rc)}")
+            raise RuntimeError(f"ffa_attention failed: {self.capi.status_string(rc)}")
 
     def mean_bytes(self, steps):
-        return sum(algorithmic_bytes(self.B, self.H, self.Dh, self.t_of(i)) for i in range(steps)) / steps
+        return sum(algorithmic_bytes(self.B, self.H, self.Dh, self.t_of(i), self.elem) for i in range(steps)) / steps
 
 
 def time_region(torch, fn):
@@ -184,7 +192,7 @@ def run_ext(wl, steps, warmup):
     torch = wl.torch
     from fastforwardattention_amd import FastForwardAttn
     B, H, Dh = wl.B, wl.H, wl.Dh
-    dummy = torch.zeros(B, H, 1, Dh, dtype=torch.float16, device="cuda:0")
+    dummy = torch.zeros(B, H, 1, Dh, dtype=wl.tdtype, device="cuda:0")
     obj = FastForwardAttn(dummy, dummy, wl.Lmax, wl.use_default)  # its own caches are unused
     def step(i):
         r, l = i % wl.ring, i % wl.layers
@@ -199,37 +207,39 @@ def run_ext(wl, steps, warmup):
 
 
 def parity_check(wl):
-    """The workload's whole decode loop on one layer cache, untimed: fp16 kernel output through
-    the C ABI (the library's own launch plan at every step) against fp32 torch on the GPU
-    (softmax(q K^T scale) V over the upcast fp16 inputs).  Returns the worst max-abs error."""
+    """The workload's whole decode loop on one layer cache, untimed: kernel output through the
+    C ABI (the library's own launch plan at every step) against fp32 torch on the GPU
+    (softmax(q K^T scale) V over the upcast inputs).  Returns the worst max-abs error; the
+    tolerance is 1e-3 for fp16 inputs and 1e-6 for fp32 inputs."""
     torch, capi, lib = wl.torch, wl.capi, wl.lib
     B, H, Dh, L, Lmax, gen = wl.B, wl.H, wl.Dh, wl.prompt, wl.Lmax, wl.gen
-    dev = "cuda:0"
+    dev, tdt, x = "cuda:0", wl.tdtype, 16 // wl.elem
+    tol = 1e-3 if wl.dtype == "f16" else 1e-6
     g = torch.Generator(device=dev).manual_seed(1)
-    K = (torch.randn(B, H, L, Dh, device=dev, generator=g) * 0.5).half()
-    V = (torch.randn(B, H, L, Dh, device=dev, generator=g) * 0.5).half()
-    kc = torch.empty(B, H, Dh // 8, Lmax, 8, dtype=torch.float16, device=dev)
-    vc = torch.empty(B, H, Lmax, Dh, dtype=torch.float16, device=dev)
-    capi.check(lib.ffa_init_cache_f16(kc.data_ptr(), vc.data_ptr(), K.data_ptr(), V.data_ptr(),
-                                      B, L, Lmax, Dh, H, None), "ffa_init_cache_f16")
+    K = (torch.randn(B, H, L, Dh, device=dev, generator=g) * 0.5).to(tdt)
+    V = (torch.randn(B, H, L, Dh, device=dev, generator=g) * 0.5).to(tdt)
+    kc = torch.empty(B, H, Dh // x, Lmax, x, dtype=tdt, device=dev)
+    vc = torch.empty(B, H, Lmax, Dh, dtype=tdt, device=dev)
+    capi.check(wl.fn_init(kc.data_ptr(), vc.data_ptr(), K.data_ptr(), V.data_ptr(), B, L, Lmax, Dh, H, None),
+               "ffa_init_cache")
     Kf = torch.zeros(B * H, Lmax, Dh, device=dev)
     Vf = torch.zeros(B * H, Lmax, Dh, device=dev)
     Kf[:, :L], Vf[:, :L] = K.float().reshape(B * H, L, Dh), V.float().reshape(B * H, L, Dh)
-    out = torch.empty(B, H, Dh, dtype=torch.float16, device=dev)
+    out = torch.empty(B, H, Dh, dtype=tdt, device=dev)
     worst = 0.0
     for i in range(gen):
         t = L + i
-        q, k, v = (torch.randn(B, H, Dh, device=dev, generator=g).half() for _ in range(3))
+        q, k, v = (torch.randn(B, H, Dh, device=dev, generator=g).to(tdt) for _ in range(3))
         plan = wl.plan_for(t)
-        capi.check(lib.ffa_attention_f16(B, H, Dh, Lmax, wl.scale, t, q.data_ptr(), k.data_ptr(), v.data_ptr(),
-                                         kc.data_ptr(), vc.data_ptr(), out.data_ptr(), None, 0.0, C.byref(plan), 1,
-                                         wl.ws.data_ptr(), wl.ws_bytes, None), "ffa_attention_f16")
+        capi.check(wl.fn_attn(B, H, Dh, Lmax, wl.scale, t, q.data_ptr(), k.data_ptr(), v.data_ptr(),
+                              kc.data_ptr(), vc.data_ptr(), out.data_ptr(), None, 0.0, C.byref(plan), 1,
+                              wl.ws.data_ptr(), wl.ws_bytes, None), "ffa_attention")
         Kf[:, t], Vf[:, t] = k.float().reshape(B * H, Dh), v.float().reshape(B * H, Dh)
         w = torch.softmax(torch.bmm(q.float().reshape(B * H, 1, Dh), Kf[:, :t + 1].transpose(1, 2)) * wl.scale, -1)
         ref = torch.bmm(w, Vf[:, :t + 1]).reshape(B, H, Dh)
         worst = max(worst, float((out.float() - ref).abs().max()))
-    return {"max_abs_err": worst, "tolerance": 1e-3, "steps": gen, "ok": worst <= 1e-3,
-            "reference": "fp32 torch bmm/softmax/bmm on the GPU over the upcast fp16 inputs, every step"}
+    return {"max_abs_err": worst, "tolerance": tol, "steps": gen, "ok": worst <= tol,
+            "reference": "fp32 torch bmm/softmax/bmm on the GPU over the upcast inputs, every step"}
 
 
 def cpu_baseline(wl, budget_s=15.0, max_steps=64):
@@ -427,7 +437,7 @@ def run_init_cache_bench():
 
 def run_suite(args):
     """Every BASELINE.json configuration that fits one GPU, one JSON object per line."""
-    for name in ["opt1.3b_b10", "opt1.3b_b5", "opt1.3b_b2", "opt1.3b_b1", "opt2.7b_b10", "gptj_b8",
+    for name in ["opt1.3b_b10", "opt1.3b_b5", "opt1.3b_b2", "opt1.3b_b1", "opt1.3b_b10_f32", "opt2.7b_b10", "gptj_b8",
                  "long_b1_1k", "long_b1_2k", "long_b1_4k", "long_b1_8k", "long_b1_16k"]:
         for use_default in (False, True):
             wl = Workload(name, use_default=use_default)
@@ -549,8 +559,8 @@ def main():
         "ms_per_step": round(us_step / 1e3, 6), "us_per_step": round(us_step, 3),
         "tokens_per_s": round(wl.B / (us_step * 1e-6), 1),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "f16", "accumulate_dtype": "f32", "data": "synthetic",
-        "config": {"workload": f"{args.workload}: B={wl.B} H={wl.H} Dh={wl.Dh} fp16 prompt={wl.prompt} "
+        "dtype": wl.dtype, "accumulate_dtype": "f32", "data": "synthetic",
+        "config": {"workload": f"{args.workload}: B={wl.B} H={wl.H} Dh={wl.Dh} {wl.dtype} prompt={wl.prompt} "
                                f"t={wl.prompt}->{wl.prompt + min(wl.gen, -(-steps // wl.layers))} p=0 "
                                f"scale={wl.scale}; step = one attention call on one of {wl.layers} "
                                "independent layer caches",

@@ -162,4 +162,7 @@ def test_hook_with_hip_engine(family, dtype, tol):
         assert float((got - want).abs().max()) < tol
         import ff_attention
         assert all(isinstance(layer.engine, ff_attention.FastForwardAttn) for layer in cache.layers)
+    # a threshold far below every probability: the pruning kernels must reproduce the exact logits
+    got, _ = teacher_forced_logits(model, ids, mask, steps, hf.FFACache(max_new_tokens=steps, prob_thresh=1e-7))
+    assert float((got - want).abs().max()) < tol
     hf.disable(model)
