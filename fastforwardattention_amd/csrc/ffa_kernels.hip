@@ -9,7 +9,8 @@
 //   v_cache [B,H,Lmax,Dh]: a row is Dh*sizeof(T) bytes = LPR 16-byte chunks.  Lane l owns
 //     chunk (l % LPR) of row (l / LPR) of each group of RPI = 64/LPR consecutive rows, so
 //     a load instruction again covers 1 KiB contiguous.
-// A 64-key tile is NCH = Dh/x load instructions for K and NCH for V.  The probabilities
+// A 64-key tile is NCH = Dh/x load instructions for K and LPR (= NCH rounded up to a power of
+// two; Dh = 80 has 10 or 20 chunks on 16 or 32 lanes) for V.  The probabilities
 // computed in the K mapping (one key per lane) reach the V mapping (one row per LPR lanes)
 // through a 256-byte LDS stage per wave.
 //
