@@ -1013,14 +1013,14 @@ __global__ void __launch_bounds__(256) ffa_init_cache_kernel(uint4* __restrict__
 #pragma unroll
     for (int j = 0; j < PER; ++j) {
         const int i = min((int)threadIdx.x + j * 256, n - 1);
-        kv[j] = ks[i];
-        vv[j] = vs[i];
+        kv[j] = ld16(&ks[i]);
+        vv[j] = ld16(&vs[i]);
     }
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int j = 0; j < PER; ++j) {
         const int i = threadIdx.x + j * 256;
-        if (i < n) vd[i] = vv[j];                                            // V: contiguous copy
+        if (i < n) st16_stream(&vd[i], vv[j]);                               // V: contiguous copy
         if (i < TK * NCH) s_tile[(i % NCH) * (TK + 1) + i / NCH] = kv[j];   // K: [key][chunk] -> [chunk][key]
     }
     __syncthreads();
@@ -1028,7 +1028,7 @@ __global__ void __launch_bounds__(256) ffa_init_cache_kernel(uint4* __restrict__
     for (int j = 0; j < PER; ++j) {
         const int i = threadIdx.x + j * 256;
         const int c = i / TK, key = i % TK;
-        if (c < NCH && key * NCH < n) kd[(size_t)c * Lmax + key] = s_tile[c * (TK + 1) + key];
+        if (c < NCH && key * NCH < n) st16_stream(&kd[(size_t)c * Lmax + key], s_tile[c * (TK + 1) + key]);
     }
 }
 
