@@ -435,6 +435,68 @@ def run_init_cache_bench():
     return {"kernel": "ffa_init_cache_kernel (cache construction, fp16)", "results": res}
 
 
+def run_hf_end_to_end(B=10, prompt=1000, new_tokens=128):
+    """The reference's end-to-end setting in miniature (summarize.py: OPT with a left-padded batch,
+    greedy decoding): an OPT-1.3b-shaped model with random weights (nothing is downloaded), prompt
+    of `prompt` tokens, `new_tokens` decode steps; wall time per generated token with transformers'
+    own cache and attention against the FFACache hook.  Reported beside the kernel figures; the
+    projections and MLPs of the model dominate a decode step, the attention call is what changes."""
+    import torch
+    import transformers
+    from fastforwardattention_amd import hf
+    cfg = transformers.OPTConfig(vocab_size=50272, hidden_size=2048, num_hidden_layers=24, ffn_dim=8192,
+                                 num_attention_heads=32, max_position_embeddings=2048, word_embed_proj_dim=2048,
+                                 dropout=0.0, attention_dropout=0.0)
+    torch.manual_seed(0)
+    with torch.device("cuda:0"):
+        model = transformers.OPTForCausalLM(cfg).half().eval()
+    g = torch.Generator(device="cuda:0").manual_seed(0)
+    ids = torch.randint(4, 50000, (B, prompt), device="cuda:0", generator=g)
+    mask = torch.ones_like(ids)
+    mask[1::2, :37] = 0                      # every other sample is left-padded by 37 tokens
+    kw = dict(attention_mask=mask, max_new_tokens=new_tokens, min_new_tokens=new_tokens, do_sample=False,
+              pad_token_id=1)
+
+    def timed(**extra):
+        with torch.no_grad():
+            model.generate(ids, **{**kw, **extra, "max_new_tokens": 4, "min_new_tokens": 4})   # warm-up
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            model.generate(ids, **{**kw, **extra, "max_new_tokens": 1, "min_new_tokens": 1})   # prompt pass + 1 token
+            torch.cuda.synchronize()
+            t1 = time.perf_counter()
+            out = model.generate(ids, **{**kw, **extra})
+            torch.cuda.synchronize()
+            t2 = time.perf_counter()
+        return out, ((t2 - t1) - (t1 - t0)) * 1e3 / (new_tokens - 1)
+
+    res = {}
+    for impl in ("sdpa", "eager"):
+        model.config._attn_implementation = impl
+        ref_out, ms = timed()
+        res[f"transformers_{impl}_ms_per_token"] = round(ms, 3)
+    hf.enable(model)
+    outs = {}
+    for name, default in (("ffa_tuned", False), ("ffa_default_launch", True)):
+        with torch.no_grad():
+            # a cache object serves one generate() call: build a new one per call
+            def run(n):
+                return model.generate(ids, **{**kw, "max_new_tokens": n, "min_new_tokens": n},
+                                      past_key_values=hf.FFACache(max_new_tokens=n, use_default_kernel_launch=default))
+            run(4)
+            torch.cuda.synchronize()
+            t0 = time.perf_counter(); run(1); torch.cuda.synchronize()
+            t1 = time.perf_counter(); out = run(new_tokens); torch.cuda.synchronize()
+            t2 = time.perf_counter()
+        res[f"{name}_ms_per_token"] = round(((t2 - t1) - (t1 - t0)) * 1e3 / (new_tokens - 1), 3)
+        outs[name] = out
+    hf.disable(model)
+    res["same_tokens_as_transformers_eager"] = bool(torch.equal(outs["ffa_tuned"], ref_out))
+    res["matching_token_fraction"] = round(float((outs["ffa_tuned"] == ref_out).double().mean().item()), 6)
+    return {"workload": f"OPT-1.3b-shaped random model, fp16, B={B}, prompt {prompt} (odd samples left-padded by 37), "
+                        f"{new_tokens} greedy tokens; per-token time excludes the prompt pass", **res}
+
+
 def run_suite(args):
     """Every BASELINE.json configuration that fits one GPU, one JSON object per line."""
     for name in ["opt1.3b_b10", "opt1.3b_b5", "opt1.3b_b2", "opt1.3b_b1", "opt1.3b_b10_f32", "opt2.7b_b10", "gptj_b8",
@@ -500,6 +562,8 @@ def main():
     ap.add_argument("--plan", default=None, help="kind,waves,tiles_per_split[,combine[,whole_heads]] (kind: 0 workgroup, 1 split; combine: 0 fused, 1 kernel)")
     ap.add_argument("--legs", default="graph,capi,ext", help="comma list of graph,capi,ext")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--hf-end-to-end", action="store_true",
+                    help="only: decode an OPT-1.3b-shaped random model with and without the FFACache hook")
     ap.add_argument("--no-parity", action="store_true", help="skip the untimed every-step parity check")
     ap.add_argument("--suite", action="store_true",
                     help="run every BASELINE configuration (tuned and default launch) and the pruned sweep; "
@@ -531,6 +595,9 @@ def main():
         return
     if args.init_cache:
         print(json.dumps(run_init_cache_bench()))
+        return
+    if args.hf_end_to_end:
+        print(json.dumps(run_hf_end_to_end()))
         return
 
     plan_override = tuple(int(x) for x in args.plan.split(",")) if args.plan else None
