@@ -160,3 +160,45 @@ def test_full_size_iterative_decode_every_step(name, dtype, tol, B, H, Dh, L, ge
     kc, vc = ffa.get_cache()
     assert torch.equal(vc.float().reshape(B * H, Lmax, Dh), Vf)
     assert torch.equal(kc.permute(0, 1, 3, 2, 4).reshape(B * H, Lmax, Dh).float(), Kf)
+
+
+@pytest.mark.parametrize("default_launch", [False, True])
+def test_decode_steps_replay_from_a_captured_graph(default_launch):
+    """Four consecutive decode steps captured into one HIP graph (static q/k/v buffers) and
+    replayed with fresh inputs, eager work and synchronisations in between: every replay must
+    reproduce what eager calls give for the same inputs (the library records kernels only: no
+    memsets, no allocations of its own in the step)."""
+    from ff_attention import FastForwardAttn as FFA
+    B, H, Dh, L, steps = 4, 32, 64, 700, 4         # 128 pairs: the split kernel with cross-workgroup merges
+    g = torch.Generator().manual_seed(5)
+    K = torch.randn(B, H, L, Dh, generator=g).half().cuda()
+    V = torch.randn(B, H, L, Dh, generator=g).half().cuda()
+    ffa_graph = FFA(K, V, L + steps, default_launch)
+    ffa_eager = FFA(K, V, L + steps, default_launch)
+    qs, ks, vs = (torch.zeros(steps, B, H, 1, Dh, dtype=torch.float16, device="cuda") for _ in range(3))
+    outs = torch.zeros(steps, B, H, Dh, dtype=torch.float16, device="cuda")
+
+    def run_steps(ffa, dst):
+        for i in range(steps):
+            dst[i].copy_(ffa.attention(qs[i], ks[i], vs[i], 0.125, L + i, 0))
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        run_steps(ffa_graph, outs)                  # warm-up on the capture stream
+    side.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        run_steps(ffa_graph, outs)
+    for replay in range(3):
+        for buf in (qs, ks, vs):
+            buf.copy_(torch.randn(buf.shape, generator=g).half())
+        graph.replay()
+        torch.cuda.synchronize()
+        got = outs.clone()
+        want = torch.zeros_like(outs)
+        run_steps(ffa_eager, want)                  # eager work between the replays
+        torch.cuda.synchronize()
+        assert float((got.float() - want.float()).abs().max()) <= 1e-3, replay
+        for a, b in zip(ffa_graph.get_cache(), ffa_eager.get_cache()):
+            assert torch.equal(a, b)
