@@ -584,6 +584,8 @@ def main():
         print("bench.py: no GPU visible; the hot path has no CPU fallback.", file=sys.stderr)
         sys.exit(3)
 
+    from fastforwardattention_amd import _build
+    _build.ensure_built()
     if args.calibrate_copy:
         run_copy_calibration()
         return

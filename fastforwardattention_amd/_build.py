@@ -72,6 +72,15 @@ def build_all() -> None:
     build_ext()
 
 
+def ensure_built() -> None:
+    """Build whatever is missing, and only that (tests, the smoke run and the benchmark load
+    what is already built)."""
+    if not os.path.exists(LIB_PATH):
+        build_lib()
+    if not os.path.exists(EXT_PATH):
+        build_ext()
+
+
 if __name__ == "__main__":
     if "--lib" in sys.argv:
         build_lib()

@@ -15,6 +15,8 @@ if _EXT_DIR not in sys.path:
 
 def pytest_configure(config):
     config.addinivalue_line("markers", "gpu: needs a real MI355X (run with -m gpu on the GPU box)")
+    from fastforwardattention_amd import _build
+    _build.ensure_built()      # loads what is built; compiles only what is missing
 
 
 def _have_gpu() -> bool:
