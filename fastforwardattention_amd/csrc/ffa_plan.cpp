@@ -102,8 +102,8 @@ int plan_launch(int precision, int B, int H, int Dh, int t, float p, int use_def
     //    never so many that a wave is left without a tile.
     //  - Long sequences with at least one pair per CU: the one-workgroup kernel with 16 waves
     //    (70 VGPRs, two workgroups = 32 waves resident per CU, separate K and V phases) streams
-    //    3-6 % faster than the split kernel (8192 keys: 256 pairs 104 vs 111 us, 512 pairs
-    //    205 vs 214 us, 1024 pairs 395 vs 412 us; 4096 keys: 95 vs 98, 184 vs 191 us); below
+    //    up to 8 % faster than the split kernel (8192 keys: 256 pairs 91 vs 99 us, 512 pairs
+    //    181 vs 193 us, 1024 pairs 353 vs 373 us; 4096 keys: 84 vs 85, 167 vs 170 us); below
     //    4096 keys the split kernel is ahead.
     if (bh >= cus && ntiles >= 64 && fits_wg) {
         fill(plan, FFA_LAUNCH_WORKGROUP, 16, 1, ntiles);
@@ -126,7 +126,7 @@ int plan_launch(int precision, int B, int H, int Dh, int t, float p, int use_def
     n_splits = ceil_div(ntiles, tps);
     if (n_splits == 1) whole = bh;  // nothing left to split: plain one-workgroup-per-pair
     // Between CUs/2 and CUs pairs nothing can be cut without doubling up CUs; the idle CUs
-    // are made up for with 8 waves per workgroup (160 pairs, 1000 keys: 9.8 vs 10.1 us).
+    // are made up for with 8 waves per workgroup (160 pairs, 1000 keys: 9.3 vs 9.8 us).
     if (n_splits == 1 && bh < cus) {
         fill(plan, FFA_LAUNCH_SPLIT, wg_waves_for(ntiles, 8), 1, ntiles);
         plan->whole_heads = bh;
