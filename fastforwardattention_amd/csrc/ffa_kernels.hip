@@ -277,11 +277,10 @@ __device__ __forceinline__ void queue_drain(float (&acc)[Elem<T>::X], SurvivorQu
 template <typename T, int DH, int NW>
 __device__ __forceinline__ void finish_piece(const DecodeParams& P, int bh, int split, int n_splits,
                                              float (&acc)[Elem<T>::X], float m_run, float l_run,
-                                             float (*s_acc)[DH], float* s_m, float* s_l, int* s_last_p) {
+                                             float (*s_acc)[DH], float* s_m, float* s_l) {
     using G = Geo<T, DH>;
     constexpr int X = G::X, LPR = G::LPR, NCH = G::NCH;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    int& s_last = *s_last_p;
 #ifdef FFA_TRACE
     unsigned long long* ffa_row = nullptr;
     if (P.trace) ffa_row = P.trace + (size_t)__builtin_amdgcn_readfirstlane(blockIdx.x * NW + wave) * 16;
@@ -336,14 +335,18 @@ __device__ __forceinline__ void finish_piece(const DecodeParams& P, int bh, int 
         return;
     }
 
-    // ---- publish the partial; the last workgroup to arrive merges all splits ----
+    // ---- publish the partial; the last wave to arrive merges all splits ----
     // No device-scope fence here: on this part such a fence writes back / invalidates a
     // whole L2 and costs far more than the kernel itself.  Instead every word that crosses
     // workgroups is moved with device-scope atomic accesses, which the hardware performs
-    // at the level all XCDs share, so nothing needs flushing.  Order: every thread waits
-    // until its own published stores have been acknowledged (wait_published) and only then
-    // enters the workgroup barrier; the arrival counter is bumped after the barrier, and the
-    // merging workgroup reads the partials only after it has seen the final count.
+    // at the level all XCDs share, so nothing needs flushing.
+    // The protocol runs per wave, without further workgroup barriers: the waves that hold
+    // output elements (the first ceil(Dh/64)) each publish theirs, wait until the stores have
+    // been acknowledged (wait_published), and only then bump the pair's arrival counter; the
+    // wave that sees the final count -- n_splits pieces x publishing waves -- knows that
+    // every partial of the pair is in memory and merges all of them.
+    constexpr int NPUB = (DH + kWave - 1) / kWave < NW ? (DH + kWave - 1) / kWave : NW;  // publishing waves
+    if (wave >= NPUB) return;
     if (tid == 0) {
         float* ml = P.ws_ml + (slot0 + split) * 2;
         publish(&ml[0], M);
@@ -351,21 +354,18 @@ __device__ __forceinline__ void finish_piece(const DecodeParams& P, int bh, int 
     }
     FFA_TP(4);
     wait_published();
-    __syncthreads();
     FFA_TP(5);
-    if (tid == 0) {
-        const unsigned prev =
-            __hip_atomic_fetch_add(&P.ws_cnt[bh], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        s_last = (prev == (unsigned)(n_splits - 1));
-    }
-    __syncthreads();
+    unsigned prev = 0;
+    if (lane == 0)
+        prev = __hip_atomic_fetch_add(&P.ws_cnt[bh], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    prev = __builtin_amdgcn_readfirstlane(prev);
     FFA_TP(6);
-    if (!s_last) return;
+    if (prev != (unsigned)(n_splits * NPUB - 1)) return;
 
     // Merge: all loads of a batch of splits are issued before any is consumed.
     const float* ml = P.ws_ml + slot0 * 2;
     constexpr int MB = 8;
-    for (int d = tid; d < DH; d += NW * 64) {
+    for (int d = lane; d < DH; d += kWave) {
         float Mg = -INFINITY, o = 0.f, Lg = 0.f;
         for (int s0 = 0; s0 < n_splits; s0 += MB) {
             float ms[MB], ls[MB], as[MB];
@@ -397,7 +397,7 @@ __device__ __forceinline__ void finish_piece(const DecodeParams& P, int bh, int 
     }
     FFA_TP(7);
     // Ready for the next launch on this stream (kernel boundaries order this store).
-    if (tid == 0) __hip_atomic_store(&P.ws_cnt[bh], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (lane == 0) __hip_atomic_store(&P.ws_cnt[bh], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 // ---------------------------------------------------------------------------------------
@@ -412,7 +412,6 @@ __global__ void __launch_bounds__(NW * 64) ffa_decode_split_kernel(const DecodeP
     __shared__ float s_acc[NW][DH];
     __shared__ float s_m[NW], s_l[NW];
     __shared__ uint4 s_q[G::Q_LDS ? NCH : 1];
-    __shared__ int s_last;
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     FFA_TP_ENTRY();
@@ -554,7 +553,7 @@ __global__ void __launch_bounds__(NW * 64) ffa_decode_split_kernel(const DecodeP
     }
     if (appends) new_token_store<NCH>(new_tok, kc_bh, vc_bh, tlen, P.Lmax, lane);
 
-    finish_piece<T, DH, NW>(P, bh, split, n_splits, acc, m_run, l_run, s_acc, s_m, s_l, &s_last);
+    finish_piece<T, DH, NW>(P, bh, split, n_splits, acc, m_run, l_run, s_acc, s_m, s_l);
 }
 
 // Merge kernel of FFA_COMBINE_KERNEL: one wave per split (b,h) pair, log-sum-exp over its
