@@ -848,7 +848,6 @@ __global__ void __launch_bounds__(NW * 64) ffa_pruned_pv_kernel(const DecodePara
     __shared__ int s_qr[NW][2 * kWave];
     __shared__ float s_acc[NW][DH];
     __shared__ unsigned s_cnt[NW];
-    __shared__ int s_last;
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int bh = blockIdx.x / P.n_splits, split = blockIdx.x % P.n_splits;
@@ -958,20 +957,20 @@ __global__ void __launch_bounds__(NW * 64) ffa_pruned_pv_kernel(const DecodePara
     }
     if (P.n_splits == 1) return;
 
-    // Same publication protocol as ffa_decode_split_kernel (device-scope relaxed atomics;
-    // stores acknowledged, then the workgroup barrier, then the arrival counter; no fences).
+    // Same per-wave publication protocol as finish_piece: the waves that hold output elements
+    // publish them, wait for the acknowledgement, bump the pair's arrival counter; the wave
+    // that sees the final count (n_splits pieces x publishing waves) sums all partials.
+    constexpr int NPUB = (DH + kWave - 1) / kWave < NW ? (DH + kWave - 1) / kWave : NW;
+    if (wave >= NPUB) return;
     wait_published();
-    __syncthreads();
-    if (tid == 0) {
-        const unsigned prev =
-            __hip_atomic_fetch_add(&P.ws_cnt[bh], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        s_last = (prev == (unsigned)(P.n_splits - 1));
-    }
-    __syncthreads();
-    if (!s_last) return;
+    unsigned prev = 0;
+    if (lane == 0)
+        prev = __hip_atomic_fetch_add(&P.ws_cnt[bh], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    prev = __builtin_amdgcn_readfirstlane(prev);
+    if (prev != (unsigned)(P.n_splits * NPUB - 1)) return;
     // All loads of a batch of pieces are issued before any is consumed.
     constexpr int MB = 8;
-    for (int d = tid; d < DH; d += NT) {
+    for (int d = lane; d < DH; d += kWave) {
         float o = 0.f;
         for (int s0 = 0; s0 < P.n_splits; s0 += MB) {
             float as[MB];
@@ -984,7 +983,7 @@ __global__ void __launch_bounds__(NW * 64) ffa_pruned_pv_kernel(const DecodePara
         }
         store_out(out, d, all_masked ? 0.f : o);
     }
-    if (tid == 0) __hip_atomic_store(&P.ws_cnt[bh], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (lane == 0) __hip_atomic_store(&P.ws_cnt[bh], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 // ---------------------------------------------------------------------------------------
