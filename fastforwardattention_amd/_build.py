@@ -35,6 +35,31 @@ HIPCC_FLAGS = [
 ]
 
 
+LIB_HASH = PKG_DIR / "libffa_hip.srchash"
+EXT_HASH = PKG_DIR / "ff_attention.srchash"
+EXT_SRC = CSRC / "torch_ffa_api.cpp"
+
+
+def _digest(files, salt) -> str:
+    import hashlib
+    h = hashlib.sha256(salt.encode())
+    for f in sorted(files):
+        h.update(f.name.encode())
+        h.update(f.read_bytes())
+    return h.hexdigest()
+
+
+def lib_source_hash() -> str:
+    """Digest of what libffa_hip.so is compiled from (sources, headers, flags)."""
+    files = [f for pat in ("*.hip", "*.cpp", "*.h", "*.inc") for f in CSRC.glob(pat) if f != EXT_SRC]
+    return _digest(files + list(INCLUDE.glob("*.h")), " ".join(HIPCC_FLAGS))
+
+
+def ext_source_hash() -> str:
+    """Digest of what the torch extension is compiled from."""
+    return _digest([EXT_SRC, *INCLUDE.glob("*.h")], "ext")
+
+
 def _run(cmd):
     print("+", " ".join(str(c) for c in cmd), flush=True)
     subprocess.run([str(c) for c in cmd], check=True)
@@ -44,6 +69,7 @@ def build_lib() -> Path:
     srcs = [CSRC / "ffa_kernels.hip", CSRC / "ffa_api.cpp", CSRC / "ffa_plan.cpp"]
     hipcc = ROCM / "bin" / "hipcc"
     _run([hipcc, *HIPCC_FLAGS, f"-I{INCLUDE}", f"-I{CSRC}", *srcs, "-o", LIB_PATH])
+    LIB_HASH.write_text(lib_source_hash())
     return LIB_PATH
 
 
@@ -64,6 +90,7 @@ def build_ext() -> Path:
            "-lffa_hip", "-lamdhip64",
            "-Wl,-rpath,$ORIGIN", f"-Wl,-rpath,{torch_lib}", f"-Wl,-rpath,{ROCM / 'lib'}"]
     _run(cmd)
+    EXT_HASH.write_text(ext_source_hash())
     return EXT_PATH
 
 
@@ -72,12 +99,20 @@ def build_all() -> None:
     build_ext()
 
 
+def _current(artefact, hash_file, digest) -> bool:
+    try:
+        return artefact.exists() and hash_file.read_text().strip() == digest()
+    except OSError:
+        return False
+
+
 def ensure_built() -> None:
-    """Build whatever is missing, and only that (tests, the smoke run and the benchmark load
-    what is already built)."""
-    if not os.path.exists(LIB_PATH):
+    """Tests, the smoke run and the benchmark load what is built.  An artefact is rebuilt when
+    it is missing or when a file it is compiled from has changed since its build (a digest of
+    the sources is kept next to each artefact), so a green run speaks for the tree as it is."""
+    if not _current(LIB_PATH, LIB_HASH, lib_source_hash):
         build_lib()
-    if not os.path.exists(EXT_PATH):
+    if not _current(EXT_PATH, EXT_HASH, ext_source_hash):
         build_ext()
 
 

@@ -40,7 +40,7 @@ class LaunchPlan(C.Structure):
                 self.n_splits, self.tiles_per_split, self.combine, self.whole_heads)
 
     def __repr__(self):
-        kind = {0: "workgroup", 1: "split"}.get(self.kind, str(self.kind))
+        kind = {0: "workgroup", 1: "split", 2: "two_pass"}.get(self.kind, str(self.kind))
         return (f"LaunchPlan(kind={kind}, waves_per_wg={self.waves_per_wg}, "
                 f"threads_per_key={self.threads_per_key}, n_splits={self.n_splits}, "
                 f"tiles_per_split={self.tiles_per_split}, combine={self.combine}, "

@@ -142,7 +142,13 @@ size_t ffa_workspace_bytes(int batch_size, int head_num, int head_dim, int max_s
 int ffa_workspace_init(void* workspace, size_t workspace_bytes, void* stream) {
     if (workspace == nullptr) return FFA_ERR_NULL_POINTER;
     if (!aligned16(workspace)) return FFA_ERR_ALIGNMENT;
-    return launch_fill_u32(static_cast<unsigned int*>(workspace), workspace_bytes / 4, 0u, stream);
+    // Only the arrival counters at the head of the workspace have to start at zero; every
+    // other word is written before it is read.  A workspace of ffa_workspace_bytes() holds at
+    // least 268 bytes per (batch, head) pair (4 of counter, 8 + 4*Dh of partials, Dh >= 64),
+    // so the counter block lies within its first 64th (plus the block's 256-byte alignment).
+    size_t bytes = align_up(workspace_bytes / 64, 256) + 256;
+    if (bytes > workspace_bytes) bytes = workspace_bytes;
+    return launch_fill_u32(static_cast<unsigned int*>(workspace), bytes / 4, 0u, stream);
 }
 
 int ffa_init_cache_f16(uint16_t* k_dst, uint16_t* v_dst, const uint16_t* k_src,

@@ -26,6 +26,8 @@
 #include <math.h>
 #include <stdint.h>
 
+#include <mutex>
+
 #include "ffa_c_api.h"
 #include "ffa_device.h"
 #include "ffa_host.h"
@@ -361,6 +363,9 @@ __device__ __forceinline__ void finish_piece(const DecodeParams& P, int bh, int 
     prev = __builtin_amdgcn_readfirstlane(prev);
     FFA_TP(6);
     if (prev != (unsigned)(n_splits * NPUB - 1)) return;
+    // Compiler-only barrier: the loads of the merge below must stay behind the counter
+    // read-modify-write (in hardware they are ordered by the branch on its returned value).
+    __atomic_signal_fence(__ATOMIC_SEQ_CST);
 
     // Merge: all loads of a batch of splits are issued before any is consumed.
     const float* ml = P.ws_ml + slot0 * 2;
@@ -968,6 +973,7 @@ __global__ void __launch_bounds__(NW * 64) ffa_pruned_pv_kernel(const DecodePara
         prev = __hip_atomic_fetch_add(&P.ws_cnt[bh], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     prev = __builtin_amdgcn_readfirstlane(prev);
     if (prev != (unsigned)(P.n_splits * NPUB - 1)) return;
+    __atomic_signal_fence(__ATOMIC_SEQ_CST);  // compiler-only: keep the merge loads behind the counter
     // All loads of a batch of pieces are issued before any is consumed.
     constexpr int MB = 8;
     for (int d = lane; d < DH; d += kWave) {
@@ -997,11 +1003,12 @@ __global__ void __launch_bounds__(256) ffa_init_cache_kernel(uint4* __restrict__
                                                              uint4* __restrict__ v_dst,
                                                              const uint4* __restrict__ k_src,
                                                              const uint4* __restrict__ v_src,
-                                                             int L, int Lmax) {
+                                                             int L, int Lmax, int tiles) {
     constexpr int PER = (TK * NCH + 255) / 256;  // chunks per thread, of K and of V
     __shared__ uint4 s_tile[NCH * (TK + 1)];  // [chunk][key], one chunk of padding per row
-    const int bh = blockIdx.y;
-    const int l0 = blockIdx.x * TK;
+    // One-dimensional grid, the tiles of a (b,h) pair adjacent: no 65535 limit on B*H.
+    const int bh = blockIdx.x / tiles;
+    const int l0 = (blockIdx.x % tiles) * TK;
     const int n = min(TK, L - l0) * NCH;  // chunks of this tile, >= NCH
     const uint4* ks = k_src + ((size_t)bh * L + l0) * NCH;
     const uint4* vs = v_src + ((size_t)bh * L + l0) * NCH;
@@ -1041,6 +1048,21 @@ static int check_launch() {
     return hipGetLastError() == hipSuccess ? FFA_OK : FFA_ERR_LAUNCH;
 }
 
+// Per-device facts, resolved once per device under a lock (several host threads may drive
+// several GPUs of one process).
+constexpr int kMaxDevices = 64;
+struct DeviceState {
+    int compute_units = 0;
+};
+static std::mutex g_dev_mutex;
+static DeviceState g_dev[kMaxDevices];
+
+static int current_device() {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) { (void)hipGetLastError(); return -1; }
+    return (dev >= 0 && dev < kMaxDevices) ? dev : -1;
+}
+
 template <typename T, int DH, int NW>
 static int launch_split(const DecodeParams& P, hipStream_t st) {
     const int n_split_heads = P.bh_total - P.n_whole;
@@ -1063,16 +1085,21 @@ template <typename T, int DH, int NW>
 static int launch_wg(const DecodeParams& P, size_t lds_bytes, hipStream_t st) {
     auto kern = ffa_decode_wg_kernel<T, DH, NW>;
     if (lds_bytes > 48 * 1024) {
-        // Raise the dynamic-LDS ceiling once per instantiation (gfx950: 160 KiB per CU).
-        static int raised = 0;
-        if (!raised) {
+        // Raise the dynamic-LDS ceiling once per instantiation and device (gfx950: 160 KiB per
+        // CU).  The attribute is a property of the loaded function, not of a stream, so the
+        // call is legal while a stream is being captured.
+        static bool raised[kMaxDevices] = {};
+        const int dev = current_device();
+        if (dev < 0) return FFA_ERR_NO_DEVICE;
+        std::lock_guard<std::mutex> lock(g_dev_mutex);
+        if (!raised[dev]) {
             if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                     hipFuncAttributeMaxDynamicSharedMemorySize,
                                     kMaxDynamicLdsBytes) != hipSuccess) {
                 (void)hipGetLastError();
                 return FFA_ERR_LAUNCH;
             }
-            raised = 1;
+            raised[dev] = true;
         }
     }
     hipLaunchKernelGGL(kern, dim3((unsigned)P.bh_total), dim3(NW * 64), lds_bytes, st, P);
@@ -1161,19 +1188,21 @@ int launch_init_cache(int precision, void* k_dst, void* v_dst, const void* k_src
     // than more loads per thread do.
     constexpr int kIc = 512;
     const int tk = nch == 10 ? 64 : nch == 20 ? 32 : kIc / nch;  // Dh = 80: 640 chunks
-    const dim3 grid((unsigned)((L + tk - 1) / tk), (unsigned)(B * H));
+    const int tiles = (L + tk - 1) / tk;
+    if ((long long)tiles * B * H > 0x7fffffffll) return FFA_ERR_SHAPE;
+    const dim3 grid((unsigned)(tiles * B * H));
     hipStream_t st = reinterpret_cast<hipStream_t>(stream);
     auto kd = reinterpret_cast<uint4*>(k_dst);
     auto vd = reinterpret_cast<uint4*>(v_dst);
     auto ks = reinterpret_cast<const uint4*>(k_src);
     auto vs = reinterpret_cast<const uint4*>(v_src);
     switch (nch) {
-        case 8: hipLaunchKernelGGL((ffa_init_cache_kernel<8, kIc / 8>), grid, dim3(256), 0, st, kd, vd, ks, vs, L, Lmax); break;
-        case 16: hipLaunchKernelGGL((ffa_init_cache_kernel<16, kIc / 16>), grid, dim3(256), 0, st, kd, vd, ks, vs, L, Lmax); break;
-        case 32: hipLaunchKernelGGL((ffa_init_cache_kernel<32, kIc / 32>), grid, dim3(256), 0, st, kd, vd, ks, vs, L, Lmax); break;
-        case 64: hipLaunchKernelGGL((ffa_init_cache_kernel<64, kIc / 64>), grid, dim3(256), 0, st, kd, vd, ks, vs, L, Lmax); break;
-        case 10: hipLaunchKernelGGL((ffa_init_cache_kernel<10, 64>), grid, dim3(256), 0, st, kd, vd, ks, vs, L, Lmax); break;
-        case 20: hipLaunchKernelGGL((ffa_init_cache_kernel<20, 32>), grid, dim3(256), 0, st, kd, vd, ks, vs, L, Lmax); break;
+        case 8: hipLaunchKernelGGL((ffa_init_cache_kernel<8, kIc / 8>), grid, dim3(256), 0, st, kd, vd, ks, vs, L, Lmax, tiles); break;
+        case 16: hipLaunchKernelGGL((ffa_init_cache_kernel<16, kIc / 16>), grid, dim3(256), 0, st, kd, vd, ks, vs, L, Lmax, tiles); break;
+        case 32: hipLaunchKernelGGL((ffa_init_cache_kernel<32, kIc / 32>), grid, dim3(256), 0, st, kd, vd, ks, vs, L, Lmax, tiles); break;
+        case 64: hipLaunchKernelGGL((ffa_init_cache_kernel<64, kIc / 64>), grid, dim3(256), 0, st, kd, vd, ks, vs, L, Lmax, tiles); break;
+        case 10: hipLaunchKernelGGL((ffa_init_cache_kernel<10, 64>), grid, dim3(256), 0, st, kd, vd, ks, vs, L, Lmax, tiles); break;
+        case 20: hipLaunchKernelGGL((ffa_init_cache_kernel<20, 32>), grid, dim3(256), 0, st, kd, vd, ks, vs, L, Lmax, tiles); break;
         default: return FFA_ERR_HEAD_DIM;
     }
     return check_launch();
@@ -1188,16 +1217,16 @@ int launch_fill_u32(unsigned int* p, size_t n, unsigned int v, void* stream) {
 }
 
 int query_compute_units() {
-    static int cached = 0;  // one device model per process
-    if (cached > 0) return cached;
-    int dev = 0;
-    if (hipGetDevice(&dev) != hipSuccess) { (void)hipGetLastError(); return -1; }
+    const int dev = current_device();
+    if (dev < 0) return -1;
+    std::lock_guard<std::mutex> lock(g_dev_mutex);
+    if (g_dev[dev].compute_units > 0) return g_dev[dev].compute_units;
     int cus = 0;
     if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) {
         (void)hipGetLastError();
         return -1;
     }
-    cached = cus;
+    g_dev[dev].compute_units = cus;
     return cus;
 }
 

@@ -104,7 +104,12 @@ int ffa_plan_launch(int precision, int batch_size, int head_num, int head_dim,
  * given problem (arrival counters, split partials, two-pass scores). */
 size_t ffa_workspace_bytes(int batch_size, int head_num, int head_dim, int max_seq_len);
 
-/* Zero the arrival counters of a fresh workspace (once, before first use). */
+/* Zero the arrival counters of a workspace of ffa_workspace_bytes() bytes (they sit at its
+ * head; the rest is left as it is).  Call once before first use, and again after any launch
+ * on the workspace that failed or was aborted: a launch that dies half-way leaves counters
+ * non-zero, and later launches would then never merge their pieces.
+ * One workspace serves one stream at a time: two launches that overlap on the same
+ * workspace race on its counters and partials. */
 int ffa_workspace_init(void* workspace, size_t workspace_bytes, void* stream);
 
 /*
