@@ -24,7 +24,7 @@ STATUS_NAMES = {
     0: "FFA_OK", 1: "FFA_ERR_NULL_POINTER", 2: "FFA_ERR_DTYPE", 3: "FFA_ERR_HEAD_DIM",
     4: "FFA_ERR_SHAPE", 5: "FFA_ERR_TIMESTEP", 6: "FFA_ERR_ALIGNMENT", 7: "FFA_ERR_WORKSPACE",
     8: "FFA_ERR_PLAN", 9: "FFA_ERR_TOO_LONG", 10: "FFA_ERR_PROB_THRESH", 11: "FFA_ERR_LAUNCH",
-    12: "FFA_ERR_NO_DEVICE",
+    12: "FFA_ERR_NO_DEVICE", 13: "FFA_ERR_SCRATCH_LIMIT",
 }
 globals().update({name: code for code, name in STATUS_NAMES.items()})   # FFA_OK, FFA_ERR_* as ints
 
@@ -66,6 +66,8 @@ SIGNATURES = {
                                _PLAN_P, _i, _vp, _sz, _vp]),
     "ffa_attention_diag": (_i, [_i, _i, _i, _i, _i, _f, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _f,
                                 _PLAN_P, _i, _vp, _sz, _vp, _vp, _vp]),
+    "ffa_attention_static_scratch": (_i, [_i, _i, _i, _i, _i, _f, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _f,
+                                          _PLAN_P, _i, _vp]),
 }
 
 _lib = None

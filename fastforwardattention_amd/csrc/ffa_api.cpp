@@ -113,6 +113,7 @@ const char* ffa_status_string(int status) {
         case FFA_ERR_PROB_THRESH: return "prob_thresh must be a finite number >= 0";
         case FFA_ERR_LAUNCH: return "HIP kernel launch failed";
         case FFA_ERR_NO_DEVICE: return "no usable HIP device";
+        case FFA_ERR_SCRATCH_LIMIT: return "the launch plan needs more scratch than the library's static 4 MiB array holds";
         default: return "unknown status";
     }
 }
@@ -182,6 +183,47 @@ int ffa_attention_diag(int precision, int batch_size, int head_num, int head_dim
     a.kept_count = kept_count; a.skip_mask = skip_mask;
     a.stream = stream;
     return run_decode(a, plan, workspace, workspace_bytes);
+}
+
+int ffa_attention_static_scratch(int precision, int batch_size, int head_num, int head_dim,
+                                  int max_seq_len, float softmax_scale, int t, const void* q,
+                                  const void* k, const void* v, void* k_cache, void* v_cache,
+                                  void* out, const int* seq_lengths, float prob_thresh,
+                                  const ffa_launch_plan* plan, int right_or_no_padding, void* stream) {
+    DecodeArgs a;
+    a.precision = precision;
+    a.B = batch_size; a.H = head_num; a.Dh = head_dim; a.Lmax = max_seq_len; a.t = t;
+    a.scale = softmax_scale; a.p = prob_thresh;
+    a.q = q; a.k = k; a.v = v;
+    a.k_cache = k_cache; a.v_cache = v_cache; a.out = out;
+    a.seq_lengths = seq_lengths;
+    a.right_or_no_padding = right_or_no_padding;
+    a.kept_count = nullptr; a.skip_mask = nullptr;
+    a.stream = stream;
+    int st = validate_decode(a);
+    if (st != FFA_OK) return st;
+    ffa_launch_plan chosen;
+    if (plan != nullptr) {
+        chosen = *plan;
+    } else {
+        st = plan_launch(precision, a.B, a.H, a.Dh, a.t, a.p, /*use_default=*/0, query_compute_units(), &chosen);
+        if (st != FFA_OK) return st;
+    }
+    st = validate_plan(chosen, precision, a.B * a.H, a.t, a.p);
+    if (st != FFA_OK) return st;
+    const size_t need = plan_workspace_bytes(chosen, a.B * a.H, a.Dh, a.Lmax);
+    if (need > kStaticScratchBytes) return FFA_ERR_SCRATCH_LIMIT;
+    void* scratch_ptr = nullptr;
+    if (need > 0) {
+        st = static_scratch_address(&scratch_ptr);
+        if (st != FFA_OK) return st;
+        // The array keeps whatever the previous call on this GPU left behind: the arrival
+        // counters of this call's pairs are cleared first (a small kernel, not a memset node,
+        // so the call may be recorded into a HIP graph).
+        st = launch_fill_u32(static_cast<unsigned int*>(scratch_ptr), (size_t)a.B * a.H, 0u, stream);
+        if (st != FFA_OK) return st;
+    }
+    return run_decode(a, &chosen, scratch_ptr, need > 0 ? kStaticScratchBytes : 0);
 }
 
 int ffa_attention_f16(int batch_size, int head_num, int head_dim, int max_seq_len,

@@ -78,6 +78,19 @@ inline size_t two_pass_workspace_bytes(int bh, int head_dim, int n_splits, int m
            align_up((size_t)bh * score_stride_for(max_seq_len) * sizeof(float), 256);
 }
 
+// Bytes of workspace one given plan needs (0 for plans that use none).
+inline size_t plan_workspace_bytes(const ffa_launch_plan& plan, int bh, int head_dim, int max_seq_len) {
+    if (plan.kind == FFA_LAUNCH_TWO_PASS) return two_pass_workspace_bytes(bh, head_dim, plan.n_splits, max_seq_len);
+    const int split_heads = bh - plan.whole_heads;
+    if (plan.kind == FFA_LAUNCH_SPLIT && plan.n_splits > 1 && split_heads > 0)
+        return workspace_bytes_for(bh, split_heads, head_dim, plan.n_splits);
+    return 0;
+}
+
+// Size of the library's own scratch array (one per GPU, held until the process ends), used by
+// ffa_attention_static_scratch in place of a caller-owned workspace.
+constexpr size_t kStaticScratchBytes = FFA_STATIC_SCRATCH_BYTES;
+
 // planner (ffa_plan.cpp)
 int plan_launch(int precision, int B, int H, int Dh, int t, float p, int use_default, int cus,
                 ffa_launch_plan* plan);
@@ -89,5 +102,8 @@ int launch_init_cache(int precision, void* k_dst, void* v_dst, const void* k_src
                       const void* v_src, int B, int H, int L, int Lmax, int Dh, void* stream);
 int launch_fill_u32(unsigned int* p, size_t n, unsigned int v, void* stream);
 int query_compute_units();
+// Device address of the current device's copy of the static scratch array (resolved once per
+// device); FFA_ERR_NO_DEVICE if the runtime cannot resolve it.
+int static_scratch_address(void** ptr);
 
 }  // namespace ffa

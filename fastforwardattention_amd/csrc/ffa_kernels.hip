@@ -34,6 +34,13 @@
 
 namespace ffa {
 
+// Scratch of the entry point that takes no workspace (ffa_attention_static_scratch): arrival
+// counters, split partials and two-pass scores live here instead of in caller-owned memory.
+// Every GPU the library runs on holds its own copy at its own address; host code never uses
+// this name as an address, only what hipGetSymbolAddress returned for the current device
+// (static_scratch_address below).
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
 struct DecodeParams {
     const void* q;
     const void* k;
@@ -1053,6 +1060,7 @@ static int check_launch() {
 constexpr int kMaxDevices = 64;
 struct DeviceState {
     int compute_units = 0;
+    void* scratch = nullptr;
 };
 static std::mutex g_dev_mutex;
 static DeviceState g_dev[kMaxDevices];
@@ -1061,6 +1069,22 @@ static int current_device() {
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess) { (void)hipGetLastError(); return -1; }
     return (dev >= 0 && dev < kMaxDevices) ? dev : -1;
+}
+
+int static_scratch_address(void** ptr) {
+    const int dev = current_device();
+    if (dev < 0 || ptr == nullptr) return FFA_ERR_NO_DEVICE;
+    std::lock_guard<std::mutex> lock(g_dev_mutex);
+    if (g_dev[dev].scratch == nullptr) {
+        void* p = nullptr;
+        if (hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)) != hipSuccess || p == nullptr) {
+            (void)hipGetLastError();
+            return FFA_ERR_NO_DEVICE;
+        }
+        g_dev[dev].scratch = p;
+    }
+    *ptr = g_dev[dev].scratch;
+    return FFA_OK;
 }
 
 template <typename T, int DH, int NW>

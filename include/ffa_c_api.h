@@ -45,7 +45,9 @@ typedef enum ffa_status {
     FFA_ERR_TOO_LONG = 9,       /* t+1 scores do not fit the LDS of an FFA_LAUNCH_WORKGROUP plan */
     FFA_ERR_PROB_THRESH = 10,   /* p is negative or NaN                                      */
     FFA_ERR_LAUNCH = 11,        /* the HIP runtime refused the launch                        */
-    FFA_ERR_NO_DEVICE = 12      /* no usable gfx950 device / HIP runtime error               */
+    FFA_ERR_NO_DEVICE = 12,     /* no usable gfx950 device / HIP runtime error               */
+    FFA_ERR_SCRATCH_LIMIT = 13  /* ffa_attention_static_scratch: the plan needs more scratch */
+                                /* than FFA_STATIC_SCRATCH_BYTES                             */
 } ffa_status;
 
 /* precision codes: the same integers the reference passes to get_launch_params
@@ -167,6 +169,29 @@ int ffa_attention_diag(int precision, int batch_size, int head_num, int head_dim
                        const int* seq_lengths, float prob_thresh, const ffa_launch_plan* plan,
                        int right_or_no_padding, void* workspace, size_t workspace_bytes,
                        uint32_t* kept_count, uint8_t* skip_mask, void* stream);
+
+/*
+ * The same step for callers that cannot allocate device memory (code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc).  No counterpart in the
+ * reference.  It takes no workspace: arrival counters, split partials and two-pass scores
+ * live in a static device array of FFA_STATIC_SCRATCH_BYTES inside the library (one copy per
+ * GPU, held until the process ends), and the call allocates and frees nothing.
+ *   - a plan (given, or chosen internally when plan == NULL) whose workspace need exceeds
+ *     FFA_STATIC_SCRATCH_BYTES is refused with FFA_ERR_SCRATCH_LIMIT before anything is
+ *     launched; FFA_LAUNCH_WORKGROUP plans need none;
+ *   - every call on a GPU shares that GPU's array: calls that overlap on one GPU (two
+ *     streams, two host threads) race; calls on one stream are ordered and safe;
+ *   - the arrival counters of the call's (batch, head) pairs are cleared by a small kernel
+ *     on `stream` ahead of the decode kernel.
+ * Arguments as ffa_attention_diag, without workspace and diagnostics.
+ */
+#define FFA_STATIC_SCRATCH_BYTES (4u << 20)
+int ffa_attention_static_scratch(int precision, int batch_size, int head_num, int head_dim,
+                                  int max_seq_len, float softmax_scale, int t, const void* q,
+                                  const void* k, const void* v, void* k_cache, void* v_cache,
+                                  void* out, const int* seq_lengths, float prob_thresh,
+                                  const ffa_launch_plan* plan, int right_or_no_padding,
+                                  void* stream);
 
 #ifdef __cplusplus
 }

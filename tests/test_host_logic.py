@@ -35,11 +35,11 @@ def test_every_declared_symbol_is_exported_and_bound(lib):
 def test_version_and_status_strings(lib):
     assert lib.ffa_api_version() == 1
     seen = set()
-    for code in range(0, 13):
+    for code in range(0, 14):
         s = capi.status_string(code)
         assert s and s != "unknown status"
         seen.add(s)
-    assert len(seen) == 13
+    assert len(seen) == 14
     assert capi.status_string(99) == "unknown status"
 
 
@@ -99,6 +99,29 @@ def test_attention_argument_validation(lib):
                  ws_bytes=1 << 20) == 8
     # one-workgroup launch whose scores cannot fit in LDS
     assert _attn(lib, t=60000, Lmax=65536, plan=wg) == 9
+
+
+def test_static_scratch_entry_validates_before_any_launch(lib):
+    """ffa_attention_static_scratch: bad arguments, malformed plans and plans whose workspace
+    need exceeds the library's static array are refused on the host, before the GPU is touched."""
+    def call(precision=16, B=2, H=4, Dh=64, Lmax=128, t=10, q=P, p=0.0, plan=None):
+        return lib.ffa_attention_static_scratch(precision, B, H, Dh, Lmax, 0.125, t, q, P, P, P, P, P, None, p,
+                                                C.byref(plan) if plan is not None else None, 1, None)
+    wg = capi.make_plan(capi.FFA_LAUNCH_WORKGROUP, 4, 1, 1)
+    assert call(precision=8, plan=wg) == capi.FFA_ERR_DTYPE
+    assert call(Dh=96, plan=wg) == capi.FFA_ERR_HEAD_DIM
+    assert call(t=128, plan=wg) == capi.FFA_ERR_TIMESTEP
+    assert call(q=None, plan=wg) == capi.FFA_ERR_NULL_POINTER
+    assert call(p=-1.0, plan=wg) == capi.FFA_ERR_PROB_THRESH
+    assert call(plan=capi.make_plan(capi.FFA_LAUNCH_WORKGROUP, 3, 1, 1)) == capi.FFA_ERR_PLAN
+    # 64 pairs x 20032 scores x 4 B = 5.1 MB of two-pass scores > 4 MiB
+    nt = 20000 // 64 + 1
+    big = capi.make_plan(capi.FFA_LAUNCH_TWO_PASS, 4, 4, -(-nt // 4))
+    assert call(B=2, H=32, Lmax=20001, t=20000, p=0.01, plan=big) == capi.FFA_ERR_SCRATCH_LIMIT
+    # split partials: 8192 pieces x (8 + 4*256) B = 8.4 MB
+    many = capi.make_plan(capi.FFA_LAUNCH_SPLIT, 1, 64, 1)
+    assert call(B=4, H=32, Dh=256, Lmax=4097, t=4095, plan=many) == capi.FFA_ERR_SCRATCH_LIMIT
+    assert "scratch" in capi.status_string(capi.FFA_ERR_SCRATCH_LIMIT)
 
 
 def test_init_cache_argument_validation(lib):
