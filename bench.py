@@ -6,19 +6,25 @@ Headline workload (BASELINE.json configs[1], B = 10): OPT-1.3b-shaped iterative 
 t = 1000 -> 1255, fresh N(0,1) q/k/v, scale 1/8, p = 0.
 
 A "step" is ONE decode-attention call: one layer's cache, one new token for the whole
-batch.  OPT-1.3b has 24 layers, so the bench keeps 24 independent caches (2.5 GB) and
-step i works on cache i % 24 at t = 1000 + (i // 24) % 256: consecutive steps never touch
-the same cache, as in a real decoder, and the 103 MB of one cache cannot be served out of
-the 256 MB last-level cache.  The default K = 6144 steps is the full 256-token decode.
+batch.  OPT-1.3b has 24 layers, so the bench keeps 24 independent caches (2.5 GB) and step i
+works on cache i % 24: consecutive steps never touch the same cache, as in a real decoder,
+and the 103 MB of one cache cannot be served out of the 256 MB last-level cache.  Whatever
+--steps K is, the K steps sample the WHOLE decode: t_i = prompt + (i * gen) // K, so K = 20
+covers t = 1000 .. 1243 and the default K = 6144 is every (layer, token) of the 256-token
+decode.  The sequence of K steps is repeated back to back until the timed region is at least
+50 ms long; `ms_per_step` is the region divided by the launches in it.
 
-Three timed legs over the same K steps, each bracketed by torch.cuda.synchronize() and
-HIP events recorded on the launch stream:
-  graph   the K launches captured once into a HIP graph and replayed (device-side rate,
-          no host gaps) -> `value`, `ms_per_step`, `roofline`
-  capi    K eager calls of ffa_attention_f16 through ctypes          -> `eager_capi_*`
-  ext     K eager calls of FastForwardAttn.attention (Python API)    -> `eager_ext_*`
+Three timed legs over the same launches, each bracketed by torch.cuda.synchronize() and HIP
+events recorded on the launch stream:
+  graph   the launches captured once into a HIP graph and replayed (device-side rate, no
+          host gaps); median of 5 replays -> `value`, `ms_per_step`, `roofline`
+  capi    eager calls of ffa_attention_f16 through ctypes          -> `eager_capi_*`
+  ext     eager calls of FastForwardAttn.attention (Python API)    -> `eager_ext_*`
 plus `cpu_baseline`: the fp32 torch restatement of the reference's torch_attn_func on the
-host cores, on a bounded sample of the same workload.
+host cores, on a bounded sample of the same workload (and BASELINE configs[0] beside it),
+and `suite`: short rows of the same measurement for the other BASELINE configurations
+(other batch sizes, the long-sequence sweep with both launches, the GPT-J shape, the pruned
+sweep); --no-suite leaves them out.
 
 Prints ONE JSON line.
 """
@@ -51,6 +57,8 @@ WORKLOADS = {
     "long_b1_4k": dict(B=1, H=32, Dh=64, prompt=4096 - 128, gen=128, scale=0.125, layers=24),
     "long_b1_2k": dict(B=1, H=32, Dh=64, prompt=2048 - 128, gen=128, scale=0.125, layers=24),
     "long_b1_1k": dict(B=1, H=32, Dh=64, prompt=1024 - 128, gen=128, scale=0.125, layers=24),
+    # BASELINE configs[0] on the GPU: one fp32 step at t = 1000 (gen = 1: every launch is that step)
+    "config1_f32_b1": dict(B=1, H=32, Dh=64, prompt=1000, gen=1, scale=0.125, layers=24, dtype="f32"),
 }
 
 
@@ -60,7 +68,7 @@ def algorithmic_bytes(B, H, Dh, t, elem=2):
 
 
 class Workload:
-    def __init__(self, name, use_default=False, plan_override=None, layers=None):
+    def __init__(self, name, use_default=False, plan_override=None, layers=None, steps=None):
         import torch
         from fastforwardattention_amd import capi
         self.torch, self.capi = torch, capi
@@ -70,6 +78,7 @@ class Workload:
         self.B, self.H, self.Dh = w["B"], w["H"], w["Dh"]
         self.prompt, self.gen, self.scale, self.layers = w["prompt"], w["gen"], w["scale"], layers or w["layers"]
         self.Lmax = self.prompt + self.gen
+        self.steps = steps or self.layers * self.gen     # launches per pass over the decode
         self.use_default = use_default
         self.plan_override = plan_override
         self.dtype = w.get("dtype", "f16")
@@ -80,7 +89,9 @@ class Workload:
         self.fn_attn = self.lib.ffa_attention_f16 if self.dtype == "f16" else self.lib.ffa_attention_f32
         x, tdt = 16 // self.elem, self.tdtype
         dev = "cuda:0"
-        B, H, Dh, L, Lmax = self.B, self.H, self.Dh, self.prompt, self.Lmax
+        # Every slot of the caches holds prompt-like data: a sampled schedule jumps over slots
+        # that a step-by-step decode would have appended, and they must not hold garbage.
+        B, H, Dh, L, Lmax = self.B, self.H, self.Dh, self.Lmax, self.Lmax
         g = torch.Generator(device=dev).manual_seed(0)
         self.kc, self.vc = [], []
         for _ in range(self.layers):
@@ -106,8 +117,17 @@ class Workload:
         self._plans = {}
         torch.cuda.synchronize()
 
+    @staticmethod
+    def describe(name):
+        """Shape of a workload without its device buffers (for the CPU baseline)."""
+        from types import SimpleNamespace
+        w = WORKLOADS[name]
+        return SimpleNamespace(name=name, B=w["B"], H=w["H"], Dh=w["Dh"], prompt=w["prompt"], gen=w["gen"],
+                               scale=w["scale"], Lmax=w["prompt"] + w["gen"])
+
     def t_of(self, i):
-        return self.prompt + (i // self.layers) % self.gen
+        """Cached keys at launch i: the `steps` launches of a pass sample the whole decode."""
+        return self.prompt + ((i % self.steps) * self.gen) // self.steps
 
     def plan_for(self, t):
         p = self._plans.get(t)
@@ -138,8 +158,13 @@ class Workload:
         if rc != 0:
             raise RuntimeError(f"ffa_attention failed: {self.capi.status_string(rc)}")
 
-    def mean_bytes(self, steps):
-        return sum(algorithmic_bytes(self.B, self.H, self.Dh, self.t_of(i), self.elem) for i in range(steps)) / steps
+    def mean_bytes(self, launches=None):
+        n = launches or self.steps
+        return sum(algorithmic_bytes(self.B, self.H, self.Dh, self.t_of(i), self.elem) for i in range(n)) / n
+
+    def t_range(self):
+        ts = [self.t_of(i) for i in range(self.steps)]
+        return min(ts), max(ts)
 
 
 def time_region(torch, fn):
@@ -153,41 +178,61 @@ def time_region(torch, fn):
     return e0.elapsed_time(e1)
 
 
-def run_graph(wl, steps, warmup):
+MIN_REGION_MS = 50.0
+
+
+def launches_for(wl, steps, warmup):
+    """Launches in one timed region: whole passes over the `steps`-launch schedule, enough of
+    them for MIN_REGION_MS at the rate the warm-up launches ran at."""
+    torch = wl.torch
+    sp = torch.cuda.current_stream().cuda_stream
+    n = max(warmup, 8)
+    for i in range(n):
+        wl.launch(i, sp)
+    torch.cuda.synchronize()
+    ms = time_region(torch, lambda: [wl.launch(i, sp) for i in range(n)])
+    passes = max(1, int(-(-MIN_REGION_MS * 1.2 // (ms / n * steps))))
+    return steps * passes
+
+
+def run_graph(wl, launches, replays=5):
+    """Returns the per-replay times (ms) of a graph holding `launches` launches."""
     torch = wl.torch
     side = torch.cuda.Stream()
     side.wait_stream(torch.cuda.current_stream())
     with torch.cuda.stream(side):          # warm-up on the capture stream, eager
-        for i in range(warmup):
+        for i in range(min(launches, 2 * wl.layers)):
             wl.launch(i, side.cuda_stream)
     side.synchronize()
     graph = torch.cuda.CUDAGraph()
     with torch.cuda.graph(graph, stream=side):
         sp = torch.cuda.current_stream().cuda_stream
-        for i in range(steps):
+        for i in range(launches):
             wl.launch(i, sp)
     graph.replay()                          # one untimed replay
     torch.cuda.synchronize()
-    best = None
-    for _ in range(3):
-        ms = time_region(torch, graph.replay)
-        best = ms if best is None else min(best, ms)
-    return best
+    return [time_region(torch, graph.replay) for _ in range(replays)]
 
 
-def run_capi(wl, steps, warmup):
+def median(xs):
+    xs = sorted(xs)
+    n = len(xs)
+    return xs[n // 2] if n % 2 else 0.5 * (xs[n // 2 - 1] + xs[n // 2])
+
+
+def run_capi(wl, launches):
     torch = wl.torch
     sp = torch.cuda.current_stream().cuda_stream
-    for i in range(warmup):
+    for i in range(min(launches, 2 * wl.layers)):
         wl.launch(i, sp)
 
     def body():
-        for i in range(steps):
+        for i in range(launches):
             wl.launch(i, sp)
     return time_region(torch, body)
 
 
-def run_ext(wl, steps, warmup):
+def run_ext(wl, launches):
     """The Python API on one object per layer, built over the same caches."""
     torch = wl.torch
     from fastforwardattention_amd import FastForwardAttn
@@ -197,11 +242,11 @@ def run_ext(wl, steps, warmup):
     def step(i):
         r, l = i % wl.ring, i % wl.layers
         return obj.attention(wl.q[r], wl.k[r], wl.v[r], wl.kc[l], wl.vc[l], wl.scale, wl.t_of(i), 0.0)
-    for i in range(warmup):
+    for i in range(min(launches, 2 * wl.layers)):
         step(i)
 
     def body():
-        for i in range(steps):
+        for i in range(launches):
             step(i)
     return time_region(torch, body)
 
@@ -296,7 +341,29 @@ def cpu_baseline(wl, budget_s=10.0, max_steps=8192):
                    f"t={L + 3}..{L + 2 + min(-(-len(times) // nlayers), span)}"
                    f"{', repeated' if len(times) > span * nlayers else ''}; {sum(times):.1f} s of CPU work), "
                    "fp32 torch bmm/softmax/bmm over a pre-allocated cache; bytes counted at 4 B/element"),
+        "config1": cpu_baseline_config1(),
     }
+
+
+def cpu_baseline_config1(budget_s=2.0):
+    """BASELINE configs[0] on the host cores: one decode-attention step, B=1, 32 heads x 64,
+    fp32, t=1000, seeded N(0,1), scale 1/8, p=0, through the restated torch_attn_func."""
+    import torch
+    from oracle.torch_attn import torch_attn_func
+    torch.manual_seed(0)
+    q = torch.randn(32, 1, 64)
+    K, V = torch.randn(32, 1001, 64), torch.randn(32, 1001, 64)     # cache + the new token
+    for _ in range(5):
+        torch_attn_func(q, K, V, 0.125)
+    times, t0 = [], time.perf_counter()
+    while time.perf_counter() - t0 < budget_s:
+        s = time.perf_counter()
+        torch_attn_func(q, K, V, 0.125)
+        times.append(time.perf_counter() - s)
+    us = 1e6 * sum(times) / len(times)
+    return {"workload": "configs[0]: B=1 H=32 Dh=64 fp32 t=1000 scale=0.125 p=0, torch_attn_func on CPU",
+            "us_per_step": round(us, 1), "GBps": round(algorithmic_bytes(1, 32, 64, 1000, 4) / us / 1e3, 2),
+            "threads": torch.get_num_threads(), "calls": len(times)}
 
 
 class PrunedWorkload:
@@ -363,7 +430,7 @@ class PrunedWorkload:
             raise RuntimeError(f"ffa_attention_diag failed: {self.capi.status_string(rc)}")
         return plan
 
-    def run(self, p, steps=64, warmup=8):
+    def run(self, p, steps=320, warmup=8):
         torch = self.torch
         sp = torch.cuda.current_stream().cuda_stream
         for i in range(warmup):
@@ -507,25 +574,54 @@ def run_hf_end_to_end(B=10, prompt=1000, new_tokens=128):
                         f"{new_tokens} greedy tokens; per-token time excludes the prompt pass", **res}
 
 
+def measure_row(name, use_default=False, steps=32, eager=True):
+    """One short row of the headline measurement for another workload: `steps` launches that
+    sample its whole decode, repeated to a region of at least MIN_REGION_MS; graph replay
+    (median of 5) and, beside it, the eager C-ABI leg."""
+    import torch
+    wl = Workload(name, use_default=use_default, steps=steps)
+    n = launches_for(wl, steps, 16)
+    us = median(run_graph(wl, n)) * 1e3 / n
+    mb = wl.mean_bytes()
+    row = {"workload": name, "use_default_kernel_launch": use_default, "B": wl.B, "H": wl.H, "Dh": wl.Dh,
+           "dtype": wl.dtype, "t_range": list(wl.t_range()), "timed_launches": n, "us_per_step": round(us, 2),
+           "GBps": round(mb / us / 1e3, 1), "hbm_frac": round(mb / us / 1e3 / HBM_PEAK_GBS, 4),
+           "plan": repr(wl.plan_for(wl.t_of(0)))}
+    if eager:
+        row["eager_capi_us_per_step"] = round(run_capi(wl, n) * 1e3 / n, 2)
+    del wl
+    torch.cuda.empty_cache()
+    return row
+
+
+SUITE_ROWS = [  # (workload, also with the default launch)
+    ("opt1.3b_b5", True), ("opt1.3b_b2", True), ("opt1.3b_b1", True),
+    ("long_b1_1k", True), ("long_b1_2k", True), ("long_b1_4k", True), ("long_b1_8k", True), ("long_b1_16k", True),
+    ("gptj_b8", True), ("config1_f32_b1", False), ("opt1.3b_b10_f32", False), ("opt2.7b_b10", False),
+]
+
+
+def run_suite_rows(full=False):
+    """The other BASELINE configurations, same method as the headline line, short rows."""
+    rows = []
+    for name, with_default in SUITE_ROWS:
+        rows.append(measure_row(name))
+        if with_default:
+            rows.append(measure_row(name, use_default=True, eager=False))
+    sweep = run_pruned_sweep(16, "library")
+    rows.append(sweep)
+    rows.append(run_pruned_sweep(1, "library"))
+    if full:
+        for B, kind in ((16, "workgroup"), (16, "two_pass"), (1, "workgroup")):
+            rows.append(run_pruned_sweep(B, kind))
+        rows.append(run_init_cache_bench())
+    return rows
+
+
 def run_suite(args):
-    """Every BASELINE.json configuration that fits one GPU, one JSON object per line."""
-    for name in ["opt1.3b_b10", "opt1.3b_b5", "opt1.3b_b2", "opt1.3b_b1", "opt1.3b_b10_f32", "opt2.7b_b10", "gptj_b8",
-                 "long_b1_1k", "long_b1_2k", "long_b1_4k", "long_b1_8k", "long_b1_16k"]:
-        for use_default in (False, True):
-            wl = Workload(name, use_default=use_default)
-            steps = wl.layers * min(wl.gen, 64)
-            ms = run_graph(wl, steps, wl.layers)
-            us = ms * 1e3 / steps
-            mb = wl.mean_bytes(steps)
-            print(json.dumps({"workload": name, "use_default_kernel_launch": use_default, "steps": steps,
-                              "t_range": [wl.t_of(0), wl.t_of(steps - 1)], "us_per_step": round(us, 2),
-                              "GBps": round(mb / us / 1e3, 1), "hbm_frac": round(mb / us / 1e3 / HBM_PEAK_GBS, 4),
-                              "plan": repr(wl.plan_for(wl.t_of(0)))}), flush=True)
-            del wl
-            import torch
-            torch.cuda.empty_cache()
-    run_pruned_sweeps()
-    print(json.dumps(run_init_cache_bench()), flush=True)
+    """Every BASELINE configuration that fits one GPU, one JSON object per line."""
+    for row in run_suite_rows(full=True):
+        print(json.dumps(row), flush=True)
 
 
 def run_copy_calibration(mib=128, reps=40):
@@ -575,6 +671,8 @@ def main():
     ap.add_argument("--hf-end-to-end", action="store_true",
                     help="only: decode an OPT-1.3b-shaped random model with and without the FFACache hook")
     ap.add_argument("--no-parity", action="store_true", help="skip the untimed every-step parity check")
+    ap.add_argument("--no-suite", action="store_true",
+                    help="leave out the short rows for the other BASELINE configurations")
     ap.add_argument("--suite", action="store_true",
                     help="run every BASELINE configuration (tuned and default launch) and the pruned sweep; "
                          "one JSON line each instead of the single headline line")
@@ -613,54 +711,65 @@ def main():
         return
 
     plan_override = tuple(int(x) for x in args.plan.split(",")) if args.plan else None
-    wl = Workload(args.workload, use_default=args.default_launch, plan_override=plan_override, layers=args.layers)
     steps, warmup = args.steps, args.warmup
+    wl = Workload(args.workload, use_default=args.default_launch, plan_override=plan_override, layers=args.layers,
+                  steps=steps)
     legs = [x for x in args.legs.split(",") if x]
-    mean_b = wl.mean_bytes(steps)
+    mean_b = wl.mean_bytes()
+    launches = launches_for(wl, steps, warmup)
 
-    res = {}
+    res, replays_us = {}, None
     if "graph" in legs:
-        res["graph"] = run_graph(wl, steps, warmup)
+        reps = run_graph(wl, launches)
+        replays_us = [round(ms * 1e3 / launches, 3) for ms in reps]
+        res["graph"] = median(reps)
     if "capi" in legs:
-        res["capi"] = run_capi(wl, steps, warmup)
+        res["capi"] = run_capi(wl, launches)
     if "ext" in legs:
-        res["ext"] = run_ext(wl, steps, warmup)
+        res["ext"] = run_ext(wl, launches)
     primary = "graph" if "graph" in res else legs[0]
-    ms = res[primary]
-    us_step = ms * 1e3 / steps
+    us_step = res[primary] * 1e3 / launches
     gbs = mean_b / (us_step * 1e-6) / 1e9
 
     plan0 = wl.plan_for(wl.t_of(0))
+    t_lo, t_hi = wl.t_range()
+    shape = f"B={wl.B} H={wl.H} Dh={wl.Dh} {wl.dtype}"
     out = {
-        "metric": "KV-cache HBM GB/s (decode attention, OPT-1.3b shape B=10, t=1000->1256)"
-                  if args.workload == "opt1.3b_b10" else f"KV-cache HBM GB/s ({args.workload})",
+        "metric": f"KV-cache HBM GB/s (decode attention, {args.workload}: {shape}, t={t_lo}->{t_hi + 1})",
         "value": round(gbs, 1), "unit": "GB/s", "n_gpus": 1, "steps": steps, "warmup": warmup,
         "ms_per_step": round(us_step / 1e3, 6), "us_per_step": round(us_step, 3),
         "tokens_per_s": round(wl.B / (us_step * 1e-6), 1),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": wl.dtype, "accumulate_dtype": "f32", "data": "synthetic",
-        "config": {"workload": f"{args.workload}: B={wl.B} H={wl.H} Dh={wl.Dh} {wl.dtype} prompt={wl.prompt} "
-                               f"t={wl.prompt}->{wl.prompt + min(wl.gen, -(-steps // wl.layers))} p=0 "
-                               f"scale={wl.scale}; step = one attention call on one of {wl.layers} "
-                               "independent layer caches",
-                   "timing_leg": primary,
+        "config": {"workload": f"{args.workload}: {shape} prompt={wl.prompt} t={t_lo}->{t_hi + 1} p=0 "
+                               f"scale={wl.scale}; step = one attention call on one of {wl.layers} independent "
+                               f"layer caches; the {steps} steps sample the decode at t_i = {wl.prompt} + "
+                               f"(i*{wl.gen})//{steps}",
+                   "timing_leg": primary, "timed_launches": launches,
+                   "timed_region_ms": round(res[primary], 3),
                    "launch_plan_at_first_step": repr(plan0)},
         "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(gbs / HBM_PEAK_GBS, 4),
                      "traffic": load_traffic(args.workload, mean_b),
                      "algorithmic_bytes_per_launch": round(mean_b),
-                     "kernel": "ffa_decode_split_kernel" if plan0.kind == 1 else "ffa_decode_wg_kernel",
+                     "kernel": {0: "ffa_decode_wg_kernel", 1: "ffa_decode_split_kernel"}.get(plan0.kind, "two-pass pair"),
                      "launch_us": round(us_step, 3)},
     }
+    if replays_us is not None:
+        out["graph_replays_us_per_step"] = replays_us
     for leg in ("capi", "ext"):
         if leg in res and leg != primary:
-            u = res[leg] * 1e3 / steps
+            u = res[leg] * 1e3 / launches
             out[f"eager_{leg}_us_per_step"] = round(u, 3)
             out[f"eager_{leg}_GBps"] = round(mean_b / (u * 1e-6) / 1e9, 1)
     if not args.no_parity:
         out["parity"] = parity_check(wl)
+    del wl
+    torch.cuda.empty_cache()
+    if not args.no_suite:
+        out["suite"] = run_suite_rows()
     if not args.no_cpu_baseline:
-        out["cpu_baseline"] = cpu_baseline(wl)
+        out["cpu_baseline"] = cpu_baseline(Workload.describe(args.workload))
     print(json.dumps(out))
     if not args.no_parity and not out["parity"]["ok"]:
         print("bench.py: parity check FAILED; the throughput above is not a valid result", file=sys.stderr)
