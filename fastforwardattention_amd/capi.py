@@ -104,9 +104,10 @@ def plan_launch(precision, B, H, Dh, t, p=0.0, use_default=False, compute_units=
     return plan
 
 
-def make_plan(kind, waves_per_wg, n_splits, tiles_per_split, combine=0, whole_heads=0) -> LaunchPlan:
+def make_plan(kind, waves_per_wg, n_splits, tiles_per_split, combine=0, whole_heads=0, threads_per_key=1) -> LaunchPlan:
     plan = LaunchPlan()
-    plan.kind, plan.waves_per_wg, plan.threads_per_key, plan.keys_per_wave = kind, waves_per_wg, 1, 64
+    plan.kind, plan.waves_per_wg = kind, waves_per_wg
+    plan.threads_per_key, plan.keys_per_wave = threads_per_key, 64 // threads_per_key
     plan.n_splits, plan.tiles_per_split, plan.combine = n_splits, tiles_per_split, combine
     plan.whole_heads = whole_heads
     return plan

@@ -43,7 +43,7 @@ int run_decode(const DecodeArgs& a, const ffa_launch_plan* user_plan, void* work
             st = plan_launch(a.precision, a.B, a.H, a.Dh, a.t, 1.f, 0, cus, &plan);
         if (st != FFA_OK) return st;
     }
-    st = validate_plan(plan, a.precision, a.B * a.H, a.t, a.p);
+    st = validate_plan(plan, a.precision, a.Dh, a.B * a.H, a.t, a.p);
     if (st != FFA_OK) return st;
     if (diag && plan.kind == FFA_LAUNCH_SPLIT) return FFA_ERR_PLAN;
 
@@ -209,7 +209,7 @@ int ffa_attention_static_scratch(int precision, int batch_size, int head_num, in
         st = plan_launch(precision, a.B, a.H, a.Dh, a.t, a.p, /*use_default=*/0, query_compute_units(), &chosen);
         if (st != FFA_OK) return st;
     }
-    st = validate_plan(chosen, precision, a.B * a.H, a.t, a.p);
+    st = validate_plan(chosen, precision, a.Dh, a.B * a.H, a.t, a.p);
     if (st != FFA_OK) return st;
     const size_t need = plan_workspace_bytes(chosen, a.B * a.H, a.Dh, a.Lmax);
     if (need > kStaticScratchBytes) return FFA_ERR_SCRATCH_LIMIT;

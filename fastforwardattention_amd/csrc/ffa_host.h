@@ -94,7 +94,8 @@ constexpr size_t kStaticScratchBytes = FFA_STATIC_SCRATCH_BYTES;
 // planner (ffa_plan.cpp)
 int plan_launch(int precision, int B, int H, int Dh, int t, float p, int use_default, int cus,
                 ffa_launch_plan* plan);
-int validate_plan(const ffa_launch_plan& plan, int precision, int bh, int t, float p);
+int validate_plan(const ffa_launch_plan& plan, int precision, int head_dim, int bh, int t, float p);
+bool tpk_supported(int precision, int head_dim, int tpk);
 
 // launchers (ffa_kernels.hip)
 int launch_decode(const DecodeArgs& a, const ffa_launch_plan& plan, const WorkspaceView& ws);

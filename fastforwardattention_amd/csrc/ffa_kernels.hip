@@ -568,6 +568,117 @@ __global__ void __launch_bounds__(NW * 64) ffa_decode_split_kernel(const DecodeP
     finish_piece<T, DH, NW>(P, bh, split, n_splits, acc, m_run, l_run, s_acc, s_m, s_l);
 }
 
+// ---------------------------------------------------------------------------------------
+// Sequence-split exact decode with TPK = 2 or 4 lanes per key.  A tile is KPT = 64 / TPK keys:
+// lane l works on key l % KPT and on the NK = NCH / TPK chunks [part*NK, part*NK + NK) of the
+// head dimension, part = l / KPT; the partial dot products of a key meet through TPK - 1
+// cross-lane exchanges.  A load instruction then covers TPK chunk rows of KPT x 16 contiguous
+// bytes (K) or still 1 KiB of consecutive V rows.  What this buys: tiles of 8 KiB / 4 KiB
+// instead of 16 KiB at Dh = 64 (twice / four times the waves can share a short sequence), and
+// at Dh = 256 a tile whose 16 loads are all in flight at once where one lane per key needs
+// four dependent groups of loads.  Pieces are cut in units of 64 keys exactly as in
+// ffa_decode_split_kernel, with which this kernel shares its epilogue.
+template <typename T, int DH, int NW, int TPK>
+__global__ void __launch_bounds__(NW * 64) ffa_decode_split_tpk_kernel(const DecodeParams P) {
+    using G = Geo<T, DH>;
+    constexpr int X = G::X, NCH = G::NCH, LPR = G::LPR, RPI = G::RPI;
+    constexpr int KPT = kWave / TPK;   // keys per tile
+    constexpr int NK = NCH / TPK;      // K loads per tile and lane
+    constexpr int NV = KPT / RPI;      // V loads per tile and lane
+    static_assert(TPK == 2 || TPK == 4, "lanes per key");
+    static_assert(NCH % TPK == 0 && KPT % RPI == 0 && NK <= 8 && NV <= 8 && NV >= 1, "tile does not fit one load group");
+
+    __shared__ float s_p[NW][KPT];
+    __shared__ float s_acc[NW][DH];
+    __shared__ float s_m[NW], s_l[NW];
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    int bh, split, n_splits;
+    if ((int)blockIdx.x < P.n_whole) {
+        bh = blockIdx.x;
+        split = 0;
+        n_splits = 1;
+    } else {
+        const int r = blockIdx.x - P.n_whole;
+        bh = P.n_whole + r / P.n_splits;
+        split = r % P.n_splits;
+        n_splits = P.n_splits;
+    }
+    const int b = bh / P.H;
+    int tlen, first;
+    step_bounds(P, b, tlen, first);
+
+    const size_t head_bytes = (size_t)P.Lmax * DH * sizeof(T);
+    char* kc_bh = reinterpret_cast<char*>(P.k_cache) + (size_t)bh * head_bytes;
+    char* vc_bh = reinterpret_cast<char*>(P.v_cache) + (size_t)bh * head_bytes;
+    const char* knew = reinterpret_cast<const char*>(P.k) + (size_t)bh * DH * sizeof(T);
+    const char* vnew = reinterpret_cast<const char*>(P.v) + (size_t)bh * DH * sizeof(T);
+    const char* qg = reinterpret_cast<const char*>(P.q) + (size_t)bh * DH * sizeof(T);
+
+    const int kl = lane % KPT, part = lane / KPT;
+    uint4 q_reg[NK];  // this lane's share of q
+#pragma unroll
+    for (int i = 0; i < NK; ++i) q_reg[i] = *reinterpret_cast<const uint4*>(qg + (part * NK + i) * 16);
+
+    // Pieces in units of 64 keys (the plan's tiles), walked in tiles of KPT keys.
+    const int ntiles64 = tlen / kWave + 1;
+    const int tps64 = n_splits == 1 ? ntiles64 : P.tiles_per_split;
+    const int ntiles = tlen / KPT + 1;  // keys 0..tlen
+    const int tile_lo = max(split * tps64 * TPK, first / KPT);
+    const int tile_hi = min(ntiles, (split + 1) * tps64 * TPK);
+    const bool appends = split == min((ntiles64 - 1) / tps64, n_splits - 1) && wave == 0;
+    NewToken new_tok;
+    if (appends) new_tok = new_token_load<NCH>(knew, vnew, lane);
+
+    const int rg = lane / LPR, dch = min(lane % LPR, NCH - 1);
+    float m_run = -INFINITY, l_run = 0.f;
+    float acc[X];
+#pragma unroll
+    for (int e = 0; e < X; ++e) acc[e] = 0.f;
+
+    for (int tile = tile_lo + wave; tile < tile_hi; tile += NW) {
+        const int key = tile * KPT + kl;
+        const bool cached = key < tlen;
+        const char* kp = cached ? kc_bh + ((size_t)(part * NK) * P.Lmax + key) * 16 : knew + part * NK * 16;
+        const size_t kstr = cached ? (size_t)P.Lmax * 16 : 16;
+        uint4 kv[NK], vv[NV];
+#pragma unroll
+        for (int i = 0; i < NK; ++i) kv[i] = ld16(kp + (size_t)i * kstr);
+#pragma unroll
+        for (int j = 0; j < NV; ++j) {
+            const int row = min(tile * KPT + j * RPI + rg, tlen);
+            vv[j] = ld16(row < tlen ? vc_bh + ((size_t)row * NCH + dch) * 16 : vnew + dch * 16);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+
+        float s = 0.f;
+#pragma unroll
+        for (int i = 0; i < NK; ++i) s = dot_chunk(kv[i], q_reg[i], s, T{});
+#pragma unroll
+        for (int off = KPT; off < kWave; off <<= 1) s += __shfl_xor(s, off);
+
+        const bool valid = key <= tlen && key >= first;
+        const float m_new = fmaxf(m_run, wave_max(valid ? s * P.scale_log2e : -INFINITY));
+        const float alpha = (m_new == -INFINITY) ? 1.f : __builtin_amdgcn_exp2f(m_run - m_new);
+        const float pr = valid ? __builtin_amdgcn_exp2f(fmaf(s, P.scale_log2e, -m_new)) : 0.f;
+        l_run = l_run * alpha + (part == 0 ? pr : 0.f);  // every key is held by TPK lanes: count it once
+        m_run = m_new;
+
+        __builtin_amdgcn_wave_barrier();
+        if (part == 0) s_p[wave][stage_slot<NV, RPI>(kl)] = pr;
+        __builtin_amdgcn_wave_barrier();
+#pragma unroll
+        for (int e = 0; e < X; ++e) acc[e] *= alpha;
+        const float* pst = &s_p[wave][rg * NV];
+#pragma unroll
+        for (int j = 0; j < NV; ++j) fma_chunk(acc, pst[j], vv[j], T{});
+        __builtin_amdgcn_wave_barrier();
+    }
+    if (appends) new_token_store<NCH>(new_tok, kc_bh, vc_bh, tlen, P.Lmax, lane);
+
+    finish_piece<T, DH, NW>(P, bh, split, n_splits, acc, m_run, l_run, s_acc, s_m, s_l);
+}
+
 // Merge kernel of FFA_COMBINE_KERNEL: one wave per split (b,h) pair, log-sum-exp over its
 // partials.
 template <typename T, int DH>
@@ -1097,6 +1208,23 @@ static int launch_split(const DecodeParams& P, hipStream_t st) {
     return check_launch();
 }
 
+template <typename T, int DH, int NW, int TPK>
+static int launch_split_tpk(const DecodeParams& P, hipStream_t st) {
+    using G = Geo<T, DH>;
+    // Combinations whose tile fits one group of at most 8 K loads and 8 V loads.
+    if constexpr (G::NCH % TPK == 0 && G::NCH / TPK <= 8 && (kWave / TPK) % G::RPI == 0 &&
+                  (kWave / TPK) / G::RPI <= 8) {
+        const int n_split_heads = P.bh_total - P.n_whole;
+        const dim3 grid((unsigned)(P.n_whole + n_split_heads * P.n_splits));
+        hipLaunchKernelGGL((ffa_decode_split_tpk_kernel<T, DH, NW, TPK>), grid, dim3(NW * 64), 0, st, P);
+        if (n_split_heads > 0 && P.n_splits > 1 && P.combine == FFA_COMBINE_KERNEL)
+            hipLaunchKernelGGL((ffa_merge_splits_kernel<T, DH>), dim3((unsigned)n_split_heads), dim3(64), 0, st, P);
+        return check_launch();
+    } else {
+        return FFA_ERR_PLAN;
+    }
+}
+
 template <typename T, int DH, int NW>
 static int launch_two_pass(const DecodeParams& P, hipStream_t st) {
     const dim3 grid((unsigned)(P.bh_total * P.n_splits));
@@ -1132,6 +1260,20 @@ static int launch_wg(const DecodeParams& P, size_t lds_bytes, hipStream_t st) {
 
 template <typename T, int DH>
 static int dispatch_waves(const DecodeParams& P, const ffa_launch_plan& plan, hipStream_t st) {
+    if (plan.kind == FFA_LAUNCH_SPLIT && plan.threads_per_key > 1) {
+        if constexpr (DH == 80) {
+            return FFA_ERR_PLAN;
+        } else {
+            const int key = plan.threads_per_key * 100 + plan.waves_per_wg;
+            switch (key) {
+                case 204: return launch_split_tpk<T, DH, 4, 2>(P, st);
+                case 208: return launch_split_tpk<T, DH, 8, 2>(P, st);
+                case 404: return launch_split_tpk<T, DH, 4, 4>(P, st);
+                case 408: return launch_split_tpk<T, DH, 8, 4>(P, st);
+                default: return FFA_ERR_PLAN;
+            }
+        }
+    }
     if (plan.kind == FFA_LAUNCH_SPLIT) {
         switch (plan.waves_per_wg) {
             case 1: return launch_split<T, DH, 1>(P, st);

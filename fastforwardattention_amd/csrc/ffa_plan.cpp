@@ -137,10 +137,26 @@ int plan_launch(int precision, int B, int H, int Dh, int t, float p, int use_def
     return FFA_OK;
 }
 
-int validate_plan(const ffa_launch_plan& plan, int precision, int bh, int t, float p) {
+// Whether the exact split kernel exists with `tpk` lanes per key for this element size and
+// head dimension: the chunks of a key must divide evenly and a tile's K loads and V loads
+// must each fit one group of at most 8.
+bool tpk_supported(int precision, int head_dim, int tpk) {
+    if (tpk == 1) return true;
+    if ((tpk != 2 && tpk != 4) || head_dim == 80) return false;
+    const int nch = head_dim * (precision / 8) / 16;
+    const int lpr = nch <= 8 ? 8 : nch <= 16 ? 16 : nch <= 32 ? 32 : 64;
+    const int rpi = kTileKeys / lpr, kpt = kTileKeys / tpk;
+    return nch % tpk == 0 && nch / tpk <= 8 && kpt % rpi == 0 && kpt / rpi <= 8;
+}
+
+int validate_plan(const ffa_launch_plan& plan, int precision, int head_dim, int bh, int t, float p) {
     const int w = plan.waves_per_wg;
     if (w != 1 && w != 2 && w != 4 && w != 8 && w != 16) return FFA_ERR_PLAN;
-    if (plan.threads_per_key != 1 || plan.keys_per_wave != kTileKeys) return FFA_ERR_PLAN;
+    const int tpk = plan.threads_per_key;
+    if ((tpk != 1 && tpk != 2 && tpk != 4) || plan.keys_per_wave != kTileKeys / tpk) return FFA_ERR_PLAN;
+    // More than one lane per key exists in the exact split kernel only, with 4 or 8 waves.
+    if (tpk > 1 && (plan.kind != FFA_LAUNCH_SPLIT || (w != 4 && w != 8) || !tpk_supported(precision, head_dim, tpk)))
+        return FFA_ERR_PLAN;
     if (plan.n_splits < 1 || plan.n_splits > kMaxSplits || plan.tiles_per_split < 1) return FFA_ERR_PLAN;
     if (plan.combine != FFA_COMBINE_FUSED && plan.combine != FFA_COMBINE_KERNEL) return FFA_ERR_PLAN;
     const int ntiles = num_tiles(t);

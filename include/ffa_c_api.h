@@ -73,10 +73,12 @@ typedef enum ffa_status {
 typedef struct ffa_launch_plan {
     int32_t kind;             /* FFA_LAUNCH_*                                              */
     int32_t waves_per_wg;     /* wave64 wavefronts per workgroup: 1, 2, 4, 8 or 16         */
-    int32_t threads_per_key;  /* lanes cooperating on one key's q.k (1 in this version)    */
-    int32_t keys_per_wave;    /* 64 / threads_per_key                                      */
+    int32_t threads_per_key;  /* lanes cooperating on one key's q.k: 1, or 2 / 4 in        */
+                              /* FFA_LAUNCH_SPLIT plans with 4 or 8 waves (head dims 64,   */
+                              /* 128 and, for 4 lanes, 256 in fp16 / 128 in fp32)          */
+    int32_t keys_per_wave;    /* 64 / threads_per_key: keys a wavefront handles per tile   */
     int32_t n_splits;         /* workgroups per (batch, head); 1 for FFA_LAUNCH_WORKGROUP  */
-    int32_t tiles_per_split;  /* 64-key tiles each split walks                             */
+    int32_t tiles_per_split;  /* 64-key blocks each split walks (whatever the tile size)   */
     int32_t combine;          /* FFA_COMBINE_*: how split partials are merged              */
     int32_t whole_heads;      /* FFA_LAUNCH_SPLIT: the first whole_heads (batch, head)     */
                               /* pairs get ONE workgroup each (no cross-workgroup merge);  */

@@ -40,6 +40,18 @@ def _plans(prec, B, H, Dh, t):
             plans.append((f"split_w{waves}_tps{tps}", capi.make_plan(capi.FFA_LAUNCH_SPLIT, waves, ns, tps)))
             plans.append((f"split_w{waves}_tps{tps}_mergekernel",
                           capi.make_plan(capi.FFA_LAUNCH_SPLIT, waves, ns, tps, capi.FFA_COMBINE_KERNEL)))
+    # 2 and 4 lanes per key (tiles of 32 and 16 keys), where the kernel exists for this shape
+    nch = Dh * (prec // 8) // 16
+    for tpk in (2, 4):
+        if Dh != 80 and nch % tpk == 0 and nch // tpk <= 8 and (tpk == 4 or nch <= 16):
+            for waves, tps in [(4, 1), (8, 2), (4, ntiles)]:
+                ns = -(-ntiles // tps)
+                if ns <= 128:
+                    plans.append((f"split_tpk{tpk}_w{waves}_tps{tps}",
+                                  capi.make_plan(capi.FFA_LAUNCH_SPLIT, waves, ns, tps, threads_per_key=tpk)))
+            plans.append((f"hybrid_tpk{tpk}_whole{B * H // 2}",
+                          capi.make_plan(capi.FFA_LAUNCH_SPLIT, 8, -(-ntiles // 2), 2, capi.FFA_COMBINE_FUSED, B * H // 2,
+                                         threads_per_key=tpk)))
     # two-pass launches (scores kernel, then weights x V): same answer at p == 0
     for waves, tps in [(1, 1), (4, 3), (8, 2), (2, ntiles)]:
         ns = -(-ntiles // tps)

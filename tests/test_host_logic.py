@@ -83,6 +83,19 @@ def test_attention_argument_validation(lib):
     assert _attn(lib, t=100, plan=capi.make_plan(capi.FFA_LAUNCH_SPLIT, 4, 1, 1)) == 8   # 1 tile < 2 needed
     assert _attn(lib, p=0.1, plan=capi.make_plan(capi.FFA_LAUNCH_SPLIT, 4, 2, 1)) == 8   # split is exact only
     assert _attn(lib, plan=capi.make_plan(capi.FFA_LAUNCH_SPLIT, 16, 2, 1)) == 8
+    # lanes per key: 1, 2 or 4; more than one only in split plans with 4 or 8 waves and only for
+    # head dimensions whose tile then fits one group of loads
+    ok = lambda **kw: _attn(lib, t=100, ws=P, ws_bytes=1 << 20, **kw)
+    assert ok(plan=capi.make_plan(capi.FFA_LAUNCH_SPLIT, 4, 2, 1, threads_per_key=3)) == 8
+    bad = capi.make_plan(capi.FFA_LAUNCH_SPLIT, 4, 2, 1, threads_per_key=2)
+    bad.keys_per_wave = 64
+    assert ok(plan=bad) == 8
+    assert ok(plan=capi.make_plan(capi.FFA_LAUNCH_WORKGROUP, 4, 1, 2, threads_per_key=2)) == 8
+    assert ok(plan=capi.make_plan(capi.FFA_LAUNCH_TWO_PASS, 4, 2, 1, threads_per_key=2)) == 8
+    assert ok(plan=capi.make_plan(capi.FFA_LAUNCH_SPLIT, 2, 2, 1, threads_per_key=2)) == 8
+    assert ok(Dh=80, plan=capi.make_plan(capi.FFA_LAUNCH_SPLIT, 4, 2, 1, threads_per_key=2)) == 8
+    assert ok(Dh=256, plan=capi.make_plan(capi.FFA_LAUNCH_SPLIT, 4, 2, 1, threads_per_key=2)) == 8      # 16 loads per tile
+    assert ok(Dh=256, precision=32, plan=capi.make_plan(capi.FFA_LAUNCH_SPLIT, 4, 2, 1, threads_per_key=4)) == 8
     # split plan without / with too small a workspace
     sp = capi.make_plan(capi.FFA_LAUNCH_SPLIT, 4, 2, 1)
     assert _attn(lib, t=100, plan=sp) == 7
