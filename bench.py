@@ -624,6 +624,224 @@ def run_suite(args):
         print(json.dumps(row), flush=True)
 
 
+# ---------------------------------------------------------------------------------------------
+# Launch-plan sweep: measures candidate launches at the BASELINE shapes and writes the table of
+# overrides that the planner compiles in (fastforwardattention_amd/csrc/ffa_plan_table.inc).
+SWEEP_SHAPES = [
+    # precision, B, H, Dh, p, max_len (the BASELINE configuration's own), cached-key counts t that are timed
+    (16, 10, 32, 64, 0.0, 1256, [1000, 1064, 1128, 1192, 1255]),
+    (16, 5, 32, 64, 0.0, 1256, [1000, 1128, 1255]),
+    (16, 2, 32, 64, 0.0, 1256, [1000, 1128, 1255]),
+    (16, 1, 32, 64, 0.0, 1256, [1000, 1128, 1255]),
+    (16, 1, 32, 64, 0.0, 1024, [896, 960]),
+    (16, 1, 32, 64, 0.0, 2048, [1920, 1984, 2047]),
+    (16, 1, 32, 64, 0.0, 4096, [3968, 4032, 4095]),
+    (16, 1, 32, 64, 0.0, 8192, [8064, 8128, 8191]),
+    (16, 1, 32, 64, 0.0, 16384, [16256, 16320, 16383]),
+    (16, 8, 16, 256, 0.0, 2256, [2000, 2128, 2255]),
+    (16, 16, 32, 64, 0.0, 8256, [8192, 8255]),
+    (16, 10, 32, 80, 0.0, 1256, [1000, 1128, 1255]),
+    (32, 10, 32, 64, 0.0, 1256, [1000, 1128, 1255]),
+    (32, 1, 32, 64, 0.0, 1001, [1000]),
+    (16, 16, 32, 64, 1e-3, 8256, [8192, 8255]),
+    (16, 1, 32, 64, 1e-3, 8256, [8192, 8255]),
+]
+SWEEP_MARGIN = 0.97   # a candidate replaces the rules' plan only when it is more than 3 % faster
+
+
+class SweepShape:
+    """Device buffers for one (precision, B, H, Dh): enough independent caches (>= 1.5 GB in all)
+    that no launch finds its data in the last-level cache.  For p > 0 the keys are peaked as in
+    BASELINE configs[4] (32 positions per head hold 4*q_dir + N(0, 0.1)) and q is fixed."""
+
+    def __init__(self, prec, B, H, Dh, p, max_len):
+        import torch
+        from fastforwardattention_amd import capi
+        self.torch, self.capi, self.lib = torch, capi, capi.load()
+        self.prec, self.B, self.H, self.Dh, self.p = prec, B, H, Dh, p
+        self.Lmax = max_len
+        elem = prec // 8
+        tdt = torch.float16 if prec == 16 else torch.float32
+        x, dev = 16 // elem, "cuda:0"
+        per_layer = 2 * B * H * self.Lmax * Dh * elem
+        self.layers = max(2, min(24, int(1.5e9 // per_layer) + 1))
+        g = torch.Generator(device=dev).manual_seed(0)
+        init = self.lib.ffa_init_cache_f16 if prec == 16 else self.lib.ffa_init_cache_f32
+        self.fn = self.lib.ffa_attention_f16 if prec == 16 else self.lib.ffa_attention_f32
+        self.q = torch.randn(B, H, Dh, device=dev, generator=g)
+        qdir = self.q / self.q.norm(dim=-1, keepdim=True)
+        self.kc, self.vc = [], []
+        for _ in range(self.layers):
+            K = torch.randn(B, H, self.Lmax, Dh, device=dev, generator=g)
+            if p > 0:
+                pos = torch.rand(B, H, self.Lmax, device=dev, generator=g).argsort(dim=-1)[:, :, :32]
+                K.scatter_(2, pos[..., None].expand(-1, -1, -1, Dh),
+                           4 * qdir[:, :, None, :] + 0.1 * torch.randn(B, H, 32, Dh, device=dev, generator=g))
+            else:
+                K *= 0.5
+            K = K.to(tdt)
+            V = (torch.randn(B, H, self.Lmax, Dh, device=dev, generator=g) * (1.0 if p > 0 else 0.5)).to(tdt)
+            kc = torch.empty(B, H, Dh // x, self.Lmax, x, dtype=tdt, device=dev)
+            vc = torch.empty(B, H, self.Lmax, Dh, dtype=tdt, device=dev)
+            capi.check(init(kc.data_ptr(), vc.data_ptr(), K.data_ptr(), V.data_ptr(), B, self.Lmax, self.Lmax, Dh, H,
+                            None), "ffa_init_cache")
+            torch.cuda.synchronize()
+            self.kc.append(kc)
+            self.vc.append(vc)
+            del K, V
+        self.q = self.q.to(tdt)
+        self.k = torch.randn(B, H, Dh, device=dev, generator=g).to(tdt)
+        self.v = torch.randn(B, H, Dh, device=dev, generator=g).to(tdt)
+        self.out = torch.empty(B, H, Dh, dtype=tdt, device=dev)
+        n = self.lib.ffa_workspace_bytes(B, H, Dh, self.Lmax)
+        self.ws = torch.zeros(n, dtype=torch.uint8, device=dev)
+        torch.cuda.synchronize()
+
+    def time_plan(self, plan, t, region_ms=4.0, repeats=3):
+        """us per launch of `plan` at t cached keys: eager launches on rotating caches, best of
+        `repeats` regions of about `region_ms`.  None if the library refuses the plan."""
+        torch = self.torch
+        sp = torch.cuda.current_stream().cuda_stream
+        scale = self.Dh ** -0.5
+
+        def go(n):
+            for i in range(n):
+                l = i % self.layers
+                rc = self.fn(self.B, self.H, self.Dh, self.Lmax, scale, t, self.q.data_ptr(), self.k.data_ptr(),
+                             self.v.data_ptr(), self.kc[l].data_ptr(), self.vc[l].data_ptr(), self.out.data_ptr(),
+                             None, self.p, C.byref(plan), 1, self.ws.data_ptr(), self.ws.numel(), sp)
+                if rc != 0:
+                    return rc
+            return 0
+        if go(self.layers) != 0:
+            torch.cuda.synchronize()
+            return None
+        torch.cuda.synchronize()
+        ms = time_region(torch, lambda: go(2 * self.layers))
+        n = max(2 * self.layers, int(region_ms / (ms / (2 * self.layers))))
+        return min(time_region(torch, lambda: go(n)) for _ in range(repeats)) * 1e3 / n
+
+
+def candidate_plans(capi, prec, B, H, Dh, t, p, cus):
+    """The rules' own plan first, then the alternatives worth timing: launch kinds, wave counts,
+    lanes per key and split factors around one workgroup per CU."""
+    ntiles, bh = t // 64 + 1, B * H
+    fits_lds = ntiles * 64 * 4 <= 140 * 1024
+    nch = Dh * (prec // 8) // 16
+    tpk_ok = lambda k: Dh != 80 and nch % k == 0 and nch // k <= 8 and (k == 4 or nch <= 16)
+    out = [("rules", capi.plan_launch(prec, B, H, Dh, t, p, False, cus, rules_only=True))]
+
+    def cut(ns):
+        ns = max(1, min(ns, ntiles, 128))
+        tps = -(-ntiles // ns)
+        return -(-ntiles // tps), tps
+
+    if p > 0:
+        if fits_lds:
+            out += [(f"workgroup w{w}", capi.make_plan(capi.FFA_LAUNCH_WORKGROUP, w, 1, ntiles)) for w in (4, 8, 16)]
+        for w in (4, 8):
+            for f in (1, 2, 4):
+                ns, tps = cut(f * cus // bh)
+                out.append((f"two_pass w{w} x{ns}", capi.make_plan(capi.FFA_LAUNCH_TWO_PASS, w, ns, tps)))
+    else:
+        geos = []
+        if bh >= cus:
+            whole = bh // cus * cus
+            rest = bh - whole
+            if rest:
+                base = -(-cus // rest)
+                geos += [(whole, base), (whole, 2 * base), (whole, max(1, base // 2))]
+            geos.append((bh, 1))
+        else:
+            geos += [(0, cus // bh), (0, max(1, cus // (2 * bh))), (0, 2 * cus // bh), (bh, 1)]
+        rule = out[0][1]
+        for w in (4, 8):
+            for whole, ns in geos:
+                ns, tps = cut(ns)
+                out.append((f"split w{w} whole{whole} x{ns}",
+                            capi.make_plan(capi.FFA_LAUNCH_SPLIT, w, ns, tps, 0, bh if ns == 1 else whole)))
+            if rule.kind == capi.FFA_LAUNCH_SPLIT:
+                for k in (2, 4):
+                    if tpk_ok(k):
+                        out.append((f"split w{w} lanes/key {k} whole{rule.whole_heads} x{rule.n_splits}",
+                                    capi.make_plan(capi.FFA_LAUNCH_SPLIT, w, rule.n_splits, rule.tiles_per_split, 0,
+                                                   rule.whole_heads, threads_per_key=k)))
+        if fits_lds:
+            out += [(f"workgroup w{w}", capi.make_plan(capi.FFA_LAUNCH_WORKGROUP, w, 1, ntiles)) for w in (4, 8, 16)]
+    seen, uniq = set(), []
+    for label, plan in out:
+        if plan.as_tuple() not in seen:
+            seen.add(plan.as_tuple())
+            uniq.append((label, plan))
+    return uniq
+
+
+def run_plan_sweep(out_path):
+    """Times every candidate at every sweep point, prints one JSON line per point and writes the
+    table.  A point keeps the rules' plan unless a candidate beats it by more than 3 % in a
+    second, longer timing of the two."""
+    import torch
+    from fastforwardattention_amd import capi
+    lib = capi.load()
+    cus = lib.ffa_device_compute_units()
+    rows = []
+    for prec, B, H, Dh, p, max_len, ts in SWEEP_SHAPES:
+        shape = SweepShape(prec, B, H, Dh, p, max_len)
+        for i, t in enumerate(ts):
+            timed = []
+            for label, plan in candidate_plans(capi, prec, B, H, Dh, t, p, cus):
+                us = shape.time_plan(plan, t)
+                if us is not None:
+                    timed.append((us, label, plan))
+            rule_us, _, rule_plan = timed[0]
+            best_us, best_label, best_plan = min(timed, key=lambda x: x[0])
+            chosen_us, chosen_label, chosen = rule_us, "rules", rule_plan
+            if best_plan.as_tuple() != rule_plan.as_tuple() and best_us < SWEEP_MARGIN * rule_us:
+                rule_us = shape.time_plan(rule_plan, t, region_ms=12.0)        # the two again, longer
+                best_us = shape.time_plan(best_plan, t, region_ms=12.0)
+                if best_us < SWEEP_MARGIN * rule_us:
+                    chosen_us, chosen_label, chosen = best_us, best_label, best_plan
+                else:
+                    chosen_us = rule_us
+            best_us = min(best_us, chosen_us)
+            # the point stands for the t halfway to its neighbours (an eighth beyond the ends)
+            lo = (ts[i - 1] + t) // 2 + 1 if i > 0 else (t - (ts[1] - t) // 2 if len(ts) > 1 else t * 7 // 8)
+            hi = (t + ts[i + 1]) // 2 if i + 1 < len(ts) else (t + (t - ts[i - 1]) // 2 if len(ts) > 1 else t * 9 // 8)
+            rows.append((prec, Dh, B * H, max(lo, 0), hi, 1 if p > 0 else 0, chosen, chosen_us, best_us, rule_us,
+                         0 if chosen_label == "rules" else 1))
+            print(json.dumps({"sweep_point": {"precision": prec, "B": B, "H": H, "Dh": Dh, "max_len": max_len, "t": t, "p": p},
+                              "t_range": [max(lo, 0), hi], "chosen": chosen_label, "chosen_us": round(chosen_us, 2),
+                              "rules_us": round(rule_us, 2), "best": best_label, "best_us": round(best_us, 2),
+                              "candidates": {label: round(us, 2) for us, label, _ in timed}}), flush=True)
+        del shape
+        torch.cuda.empty_cache()
+    dev = torch.cuda.get_device_name(0)
+    lines = [
+        "// Launch-plan table: measured choices that override the planner's rules at the points where a",
+        "// sweep on the device found a faster launch.  GENERATED -- do not edit by hand.",
+        "//   command : python bench.py --sweep-plans      (then rebuild the library)",
+        f"//   device  : {dev}, {cus} compute units",
+        "// Row: FFA_PLAN_ROW(override, precision, head_dim, pairs, t_lo, t_hi, pruned, kind, waves,",
+        "//                   threads_per_key, n_splits, whole_heads, chosen_us, best_us, rule_us)",
+        "//   override = 1: the planner launches this row's plan for t_lo <= t <= t_hi on a 256-CU device;",
+        "//   override = 0: the rules' own plan stayed within 3 % of the fastest candidate and is kept (the",
+        "//   row records the measurement).  pairs = batch * heads; pruned = 1 for prob_thresh > 0;",
+        "//   chosen_us is the time of the row's plan, best_us the fastest candidate of the sweep, rule_us",
+        "//   the time of what the rules alone launch.",
+    ]
+    for prec, Dh, pairs, lo, hi, pruned, plan, chosen_us, best_us, rule_us, override in rows:
+        lines.append(f"FFA_PLAN_ROW({override}, {prec}, {Dh}, {pairs}, {lo}, {hi}, {pruned}, {plan.kind}, "
+                     f"{plan.waves_per_wg}, {plan.threads_per_key}, {plan.n_splits}, {plan.whole_heads}, "
+                     f"{chosen_us:.2f}f, {best_us:.2f}f, {rule_us:.2f}f)")
+    with open(out_path, "w") as f:
+        f.write("\n".join(lines) + "\n")
+    print(json.dumps({"plan_table": out_path, "rows": len(rows),
+                      "overridden": sum(r[10] for r in rows)}))
+
+
+DEFAULT_SWEEP_OUT = os.path.join(ROOT, "fastforwardattention_amd", "csrc", "ffa_plan_table.inc")
+
+
 def run_copy_calibration(mib=128, reps=40):
     """A plain device-to-device copy kernel of known size, for scaling rocprofv3's
     FETCH_SIZE / WRITE_SIZE readings: every launch reads `mib` MiB and writes `mib` MiB.
@@ -676,6 +894,10 @@ def main():
     ap.add_argument("--suite", action="store_true",
                     help="run every BASELINE configuration (tuned and default launch) and the pruned sweep; "
                          "one JSON line each instead of the single headline line")
+    ap.add_argument("--sweep-plans", action="store_true",
+                    help="time candidate launch plans at the BASELINE shapes and write the planner's table of "
+                         "overrides (then rebuild the library)")
+    ap.add_argument("--sweep-out", default=DEFAULT_SWEEP_OUT, help="where --sweep-plans writes the table")
     ap.add_argument("--init-cache", action="store_true", help="only the cache-construction kernel at the BASELINE shapes")
     ap.add_argument("--pruned-sweep", action="store_true", help="only the pruned sweep (BASELINE configs[4])")
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -699,6 +921,9 @@ def main():
         return
     if args.suite:
         run_suite(args)
+        return
+    if args.sweep_plans:
+        run_plan_sweep(args.sweep_out)
         return
     if args.pruned_sweep:
         run_pruned_sweeps()

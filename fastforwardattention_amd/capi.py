@@ -56,6 +56,7 @@ SIGNATURES = {
     "ffa_status_string": (C.c_char_p, [_i]),
     "ffa_device_compute_units": (_i, []),
     "ffa_plan_launch": (_i, [_i, _i, _i, _i, _i, _f, _i, _i, _PLAN_P]),
+    "ffa_plan_launch_rules": (_i, [_i, _i, _i, _i, _i, _f, _i, _i, _PLAN_P]),
     "ffa_workspace_bytes": (_sz, [_i, _i, _i, _i]),
     "ffa_workspace_init": (_i, [_vp, _sz, _vp]),
     "ffa_init_cache_f16": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp]),
@@ -97,10 +98,10 @@ def check(status: int, what: str = "ffa call") -> None:
         raise RuntimeError(f"{what} failed: {STATUS_NAMES.get(status, status)}: {status_string(status)}")
 
 
-def plan_launch(precision, B, H, Dh, t, p=0.0, use_default=False, compute_units=256) -> LaunchPlan:
+def plan_launch(precision, B, H, Dh, t, p=0.0, use_default=False, compute_units=256, rules_only=False) -> LaunchPlan:
     plan = LaunchPlan()
-    check(load().ffa_plan_launch(precision, B, H, Dh, t, p, int(use_default), compute_units,
-                                 C.byref(plan)), "ffa_plan_launch")
+    fn = load().ffa_plan_launch_rules if rules_only else load().ffa_plan_launch
+    check(fn(precision, B, H, Dh, t, p, int(use_default), compute_units, C.byref(plan)), "ffa_plan_launch")
     return plan
 
 

@@ -120,15 +120,28 @@ const char* ffa_status_string(int status) {
 
 int ffa_device_compute_units(void) { return query_compute_units(); }
 
-int ffa_plan_launch(int precision, int batch_size, int head_num, int head_dim, int t,
-                    float prob_thresh, int use_default_kernel_launch, int compute_units,
-                    ffa_launch_plan* plan) {
+static int plan_entry(int precision, int batch_size, int head_num, int head_dim, int t, float prob_thresh,
+                      int use_default_kernel_launch, int compute_units, int use_table, ffa_launch_plan* plan) {
     if (compute_units <= 0 && !use_default_kernel_launch) {
         compute_units = query_compute_units();
         if (compute_units <= 0) return FFA_ERR_NO_DEVICE;
     }
-    return plan_launch(precision, batch_size, head_num, head_dim, t, prob_thresh,
-                       use_default_kernel_launch, compute_units, plan);
+    return plan_launch_ex(precision, batch_size, head_num, head_dim, t, prob_thresh,
+                          use_default_kernel_launch, compute_units, use_table, plan);
+}
+
+int ffa_plan_launch(int precision, int batch_size, int head_num, int head_dim, int t,
+                    float prob_thresh, int use_default_kernel_launch, int compute_units,
+                    ffa_launch_plan* plan) {
+    return plan_entry(precision, batch_size, head_num, head_dim, t, prob_thresh,
+                      use_default_kernel_launch, compute_units, /*use_table=*/1, plan);
+}
+
+int ffa_plan_launch_rules(int precision, int batch_size, int head_num, int head_dim, int t,
+                          float prob_thresh, int use_default_kernel_launch, int compute_units,
+                          ffa_launch_plan* plan) {
+    return plan_entry(precision, batch_size, head_num, head_dim, t, prob_thresh,
+                      use_default_kernel_launch, compute_units, /*use_table=*/0, plan);
 }
 
 size_t ffa_workspace_bytes(int batch_size, int head_num, int head_dim, int max_seq_len) {

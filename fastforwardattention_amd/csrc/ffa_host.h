@@ -94,6 +94,9 @@ constexpr size_t kStaticScratchBytes = FFA_STATIC_SCRATCH_BYTES;
 // planner (ffa_plan.cpp)
 int plan_launch(int precision, int B, int H, int Dh, int t, float p, int use_default, int cus,
                 ffa_launch_plan* plan);
+// use_table = 0: the rules alone (what the sweep compares the table against).
+int plan_launch_ex(int precision, int B, int H, int Dh, int t, float p, int use_default, int cus,
+                   int use_table, ffa_launch_plan* plan);
 int validate_plan(const ffa_launch_plan& plan, int precision, int head_dim, int bh, int t, float p);
 bool tpk_supported(int precision, int head_dim, int tpk);
 

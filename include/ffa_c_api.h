@@ -98,11 +98,21 @@ int ffa_device_compute_units(void);
  *   cheap enough to be called per step);  prob_thresh: the p the step will use;
  *   use_default_kernel_launch != 0 -> one workgroup per (batch, head), workgroup size by
  *   sequence length, like the FasterTransformer table at kernel_launch_utils.h:137-154;
- *   == 0 -> tuned plan for `compute_units` CUs (pass 0 to query the current device).
+ *   == 0 -> tuned plan for `compute_units` CUs (pass 0 to query the current device): rules
+ *   derived from measurements, overridden at the shapes of a sweep on the device where the
+ *   sweep found a faster launch (csrc/ffa_plan_table.inc, `python bench.py --sweep-plans`).
  */
 int ffa_plan_launch(int precision, int batch_size, int head_num, int head_dim,
                     int t, float prob_thresh, int use_default_kernel_launch,
                     int compute_units, ffa_launch_plan* plan);
+
+/* The same planner with its table of measured overrides ignored: what the rules alone would
+ * launch.  The tuned planner is rules + a table generated by a sweep on the device (the
+ * working analogue of the fitted time model at kernel_launch_utils.h:85-132); this entry is
+ * what that sweep compares its candidates against. */
+int ffa_plan_launch_rules(int precision, int batch_size, int head_num, int head_dim,
+                          int t, float prob_thresh, int use_default_kernel_launch,
+                          int compute_units, ffa_launch_plan* plan);
 
 /* Bytes of device workspace sufficient for ANY plan this library produces for the
  * given problem (arrival counters, split partials, two-pass scores). */

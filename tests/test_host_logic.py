@@ -182,7 +182,7 @@ def test_planner_consistency(prec, Dh):
             ntiles = t // 64 + 1
             for use_default in (False, True):
                 for p in (0.0, 1e-3):
-                    plan = capi.plan_launch(prec, B, H, Dh, t, p, use_default, 256)
+                    plan = capi.plan_launch(prec, B, H, Dh, t, p, use_default, 256, rules_only=True)
                     assert plan.threads_per_key == 1 and plan.keys_per_wave == 64
                     assert plan.waves_per_wg in (1, 2, 4, 8, 16)
                     assert plan.n_splits * plan.tiles_per_split >= ntiles      # every key covered
@@ -211,6 +211,48 @@ def test_planner_consistency(prec, Dh):
                         assert plan.waves_per_wg <= 8
                         if plan.n_splits == 1:
                             assert plan.whole_heads == B * H
+
+
+def _plan_table_rows():
+    path = os.path.join(ROOT, "fastforwardattention_amd", "csrc", "ffa_plan_table.inc")
+    rows = []
+    for m in re.finditer(r"^FFA_PLAN_ROW\(([^)]*)\)", open(path).read(), flags=re.M):
+        f = [x.strip().rstrip("f") for x in m.group(1).split(",")]
+        rows.append(dict(zip(["override", "precision", "Dh", "pairs", "t_lo", "t_hi", "pruned", "kind", "waves", "tpk",
+                              "n_splits", "whole"], map(int, f[:12])), chosen_us=float(f[12]), best_us=float(f[13]),
+                         rule_us=float(f[14])))
+    return rows
+
+
+def test_planner_follows_the_measured_table():
+    """Every point of the device sweep (ffa_plan_table.inc, written by `bench.py --sweep-plans`):
+    the plan the shipped planner returns there is the one the sweep chose, and that plan was
+    measured within 3 % of the fastest candidate at the point.  Rows that override the rules
+    must differ from them by more than 3 %, the others must leave the rules' plan in place."""
+    rows = _plan_table_rows()
+    assert len(rows) >= 30, "the table is generated by `python bench.py --sweep-plans` on the device"
+    for r in rows:
+        assert r["chosen_us"] <= 1.03 * r["best_us"] + 1e-6, r
+        B, H = (r["pairs"] // 32, 32) if r["pairs"] % 32 == 0 else (r["pairs"], 1)
+        p = 1e-3 if r["pruned"] else 0.0
+        for t in {r["t_lo"], (r["t_lo"] + r["t_hi"]) // 2, r["t_hi"]}:
+            got = capi.plan_launch(r["precision"], B, H, r["Dh"], t, p, False, 256)
+            rules = capi.plan_launch(r["precision"], B, H, r["Dh"], t, p, False, 256, rules_only=True)
+            if r["override"]:
+                assert r["chosen_us"] < 0.97 * r["rule_us"], r
+                assert (got.kind, got.waves_per_wg, got.threads_per_key) == (r["kind"], r["waves"], r["tpk"]), (r, got)
+                assert got.keys_per_wave == 64 // r["tpk"]
+                ntiles = t // 64 + 1
+                want_ns = -(-ntiles // -(-ntiles // min(r["n_splits"], ntiles)))
+                assert got.n_splits == want_ns and got.n_splits * got.tiles_per_split >= ntiles, (r, got)
+                assert got.whole_heads == (r["pairs"] if got.n_splits == 1 and got.kind == 1 else r["whole"])
+            else:
+                assert got.as_tuple() == rules.as_tuple(), (r, got, rules)
+            # a table measured on 256 CUs says nothing about another device
+            other = capi.plan_launch(r["precision"], B, H, r["Dh"], t, p, False, 304)
+            assert other.as_tuple() == capi.plan_launch(r["precision"], B, H, r["Dh"], t, p, False, 304,
+                                                        rules_only=True).as_tuple()
+    assert any(r["override"] for r in rows)
 
 
 def test_planner_default_follows_length_table():
