@@ -14,6 +14,7 @@ LIB_PATH = os.path.join(_PKG_DIR, "libffa_hip.so")
 FFA_OK = 0
 FFA_PRECISION_F16 = 16
 FFA_PRECISION_F32 = 32
+FFA_PRECISION_BF16 = 0xBF16
 FFA_LAUNCH_WORKGROUP = 0
 FFA_LAUNCH_SPLIT = 1
 FFA_LAUNCH_TWO_PASS = 2
@@ -24,7 +25,7 @@ STATUS_NAMES = {
     0: "FFA_OK", 1: "FFA_ERR_NULL_POINTER", 2: "FFA_ERR_DTYPE", 3: "FFA_ERR_HEAD_DIM",
     4: "FFA_ERR_SHAPE", 5: "FFA_ERR_TIMESTEP", 6: "FFA_ERR_ALIGNMENT", 7: "FFA_ERR_WORKSPACE",
     8: "FFA_ERR_PLAN", 9: "FFA_ERR_TOO_LONG", 10: "FFA_ERR_PROB_THRESH", 11: "FFA_ERR_LAUNCH",
-    12: "FFA_ERR_NO_DEVICE", 13: "FFA_ERR_SCRATCH_LIMIT",
+    12: "FFA_ERR_NO_DEVICE", 13: "FFA_ERR_SCRATCH_LIMIT", 14: "FFA_ERR_TRANSFORM",
 }
 globals().update({name: code for code, name in STATUS_NAMES.items()})   # FFA_OK, FFA_ERR_* as ints
 
@@ -47,8 +48,15 @@ class LaunchPlan(C.Structure):
                 f"whole_heads={self.whole_heads})")
 
 
+class TokenTransform(C.Structure):
+    """struct ffa_token_transform."""
+    _fields_ = [("q_bias", C.c_void_p), ("k_bias", C.c_void_p), ("v_bias", C.c_void_p),
+                ("rotary_embedding_dim", C.c_int32), ("rotary_base", C.c_float)]
+
+
 _vp, _i, _f, _sz = C.c_void_p, C.c_int, C.c_float, C.c_size_t
 _PLAN_P = C.POINTER(LaunchPlan)
+_TT_P = C.POINTER(TokenTransform)
 
 # name -> (restype, argtypes); one entry per declaration in include/ffa_c_api.h
 SIGNATURES = {
@@ -67,6 +75,8 @@ SIGNATURES = {
                                _PLAN_P, _i, _vp, _sz, _vp]),
     "ffa_attention_diag": (_i, [_i, _i, _i, _i, _i, _f, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _f,
                                 _PLAN_P, _i, _vp, _sz, _vp, _vp, _vp]),
+    "ffa_attention_ex": (_i, [_i, _i, _i, _i, _i, _f, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _f, _PLAN_P, _i, _TT_P,
+                              _vp, _sz, _vp]),
     "ffa_attention_static_scratch": (_i, [_i, _i, _i, _i, _i, _f, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _f,
                                           _PLAN_P, _i, _vp]),
 }

@@ -13,7 +13,7 @@ namespace {
 bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
 int validate_decode(const DecodeArgs& a) {
-    if (a.precision != FFA_PRECISION_F16 && a.precision != FFA_PRECISION_F32) return FFA_ERR_DTYPE;
+    if (elem_bytes(a.precision) == 0) return FFA_ERR_DTYPE;
     if (a.Dh != 64 && a.Dh != 80 && a.Dh != 128 && a.Dh != 256) return FFA_ERR_HEAD_DIM;
     if (a.B <= 0 || a.H <= 0 || a.Lmax <= 0) return FFA_ERR_SHAPE;
     if ((long long)a.B * a.H > (1ll << 24)) return FFA_ERR_SHAPE;
@@ -23,13 +23,17 @@ int validate_decode(const DecodeArgs& a) {
     if (!aligned16(a.q) || !aligned16(a.k) || !aligned16(a.v) || !aligned16(a.k_cache) ||
         !aligned16(a.v_cache) || !aligned16(a.out))
         return FFA_ERR_ALIGNMENT;
+    if (a.rotary_dim < 0 || a.rotary_dim > a.Dh || (a.rotary_dim & 1)) return FFA_ERR_TRANSFORM;
+    if (!aligned16(a.q_bias) || !aligned16(a.k_bias) || !aligned16(a.v_bias)) return FFA_ERR_TRANSFORM;
     return FFA_OK;
 }
 
-int run_decode(const DecodeArgs& a, const ffa_launch_plan* user_plan, void* workspace,
+int run_decode(const DecodeArgs& args, const ffa_launch_plan* user_plan, void* workspace,
                size_t workspace_bytes) {
+    DecodeArgs a = args;
     int st = validate_decode(a);
     if (st != FFA_OK) return st;
+    const int plan_prec = planner_precision(a.precision);
     const bool diag = a.kept_count != nullptr || a.skip_mask != nullptr;
 
     ffa_launch_plan plan;
@@ -38,18 +42,26 @@ int run_decode(const DecodeArgs& a, const ffa_launch_plan* user_plan, void* work
     } else {
         // Diagnostics do not exist in the exact split kernel: plan as for a pruned step.
         const int cus = query_compute_units();
-        st = plan_launch(a.precision, a.B, a.H, a.Dh, a.t, a.p, /*use_default=*/0, cus, &plan);
+        st = plan_launch(plan_prec, a.B, a.H, a.Dh, a.t, a.p, /*use_default=*/0, cus, &plan);
         if (st == FFA_OK && diag && plan.kind == FFA_LAUNCH_SPLIT)
-            st = plan_launch(a.precision, a.B, a.H, a.Dh, a.t, 1.f, 0, cus, &plan);
+            st = plan_launch(plan_prec, a.B, a.H, a.Dh, a.t, 1.f, 0, cus, &plan);
         if (st != FFA_OK) return st;
     }
-    st = validate_plan(plan, a.precision, a.Dh, a.B * a.H, a.t, a.p);
+    st = validate_plan(plan, plan_prec, a.Dh, a.B * a.H, a.t, a.p);
     if (st != FFA_OK) return st;
     if (diag && plan.kind == FFA_LAUNCH_SPLIT) return FFA_ERR_PLAN;
 
     WorkspaceView ws = {nullptr, nullptr, nullptr, nullptr, 0};
     const int bh = a.B * a.H;
     const int split_heads = bh - plan.whole_heads;
+    if (a.transforms_token()) {
+        // The transformed q, k, v sit behind what the plan itself uses of the workspace.
+        const size_t plan_bytes = align_up(plan_workspace_bytes(plan, bh, a.Dh, a.Lmax), 256);
+        if (workspace == nullptr || workspace_bytes < plan_bytes + token_scratch_bytes(bh, a.Dh))
+            return FFA_ERR_WORKSPACE;
+        if (!aligned16(workspace)) return FFA_ERR_ALIGNMENT;
+        a.token_scratch = static_cast<char*>(workspace) + plan_bytes;
+    }
     if (plan.kind == FFA_LAUNCH_TWO_PASS) {
         // [counters][piece (max, sum)][partial outputs][scores]
         if (workspace == nullptr ||
@@ -113,6 +125,7 @@ const char* ffa_status_string(int status) {
         case FFA_ERR_PROB_THRESH: return "prob_thresh must be a finite number >= 0";
         case FFA_ERR_LAUNCH: return "HIP kernel launch failed";
         case FFA_ERR_NO_DEVICE: return "no usable HIP device";
+        case FFA_ERR_TRANSFORM: return "bad token transform: rotary dimension must be even and within [0, head_dim], biases 16-byte aligned";
         case FFA_ERR_SCRATCH_LIMIT: return "the launch plan needs more scratch than the library's static 4 MiB array holds";
         default: return "unknown status";
     }
@@ -150,7 +163,7 @@ size_t ffa_workspace_bytes(int batch_size, int head_num, int head_dim, int max_s
     const int n_splits = max_splits_for(bh, max_seq_len);
     const size_t exact = workspace_bytes_for(bh, bh, head_dim, n_splits);
     const size_t two_pass = two_pass_workspace_bytes(bh, head_dim, n_splits, max_seq_len);
-    return exact > two_pass ? exact : two_pass;
+    return align_up(exact > two_pass ? exact : two_pass, 256) + token_scratch_bytes(bh, head_dim);
 }
 
 int ffa_workspace_init(void* workspace, size_t workspace_bytes, void* stream) {
@@ -198,6 +211,30 @@ int ffa_attention_diag(int precision, int batch_size, int head_num, int head_dim
     return run_decode(a, plan, workspace, workspace_bytes);
 }
 
+int ffa_attention_ex(int precision, int batch_size, int head_num, int head_dim, int max_seq_len,
+                     float softmax_scale, int t, const void* q, const void* k, const void* v,
+                     void* k_cache, void* v_cache, void* out, const int* seq_lengths,
+                     float prob_thresh, const ffa_launch_plan* plan, int right_or_no_padding,
+                     const ffa_token_transform* transform, void* workspace, size_t workspace_bytes,
+                     void* stream) {
+    DecodeArgs a;
+    a.precision = precision;
+    a.B = batch_size; a.H = head_num; a.Dh = head_dim; a.Lmax = max_seq_len; a.t = t;
+    a.scale = softmax_scale; a.p = prob_thresh;
+    a.q = q; a.k = k; a.v = v;
+    a.k_cache = k_cache; a.v_cache = v_cache; a.out = out;
+    a.seq_lengths = seq_lengths;
+    a.right_or_no_padding = right_or_no_padding;
+    a.kept_count = nullptr; a.skip_mask = nullptr;
+    a.stream = stream;
+    if (transform != nullptr) {
+        a.q_bias = transform->q_bias; a.k_bias = transform->k_bias; a.v_bias = transform->v_bias;
+        a.rotary_dim = transform->rotary_embedding_dim;
+        a.rotary_base = transform->rotary_base > 0.f ? transform->rotary_base : 10000.f;
+    }
+    return run_decode(a, plan, workspace, workspace_bytes);
+}
+
 int ffa_attention_static_scratch(int precision, int batch_size, int head_num, int head_dim,
                                   int max_seq_len, float softmax_scale, int t, const void* q,
                                   const void* k, const void* v, void* k_cache, void* v_cache,
@@ -219,10 +256,11 @@ int ffa_attention_static_scratch(int precision, int batch_size, int head_num, in
     if (plan != nullptr) {
         chosen = *plan;
     } else {
-        st = plan_launch(precision, a.B, a.H, a.Dh, a.t, a.p, /*use_default=*/0, query_compute_units(), &chosen);
+        st = plan_launch(planner_precision(precision), a.B, a.H, a.Dh, a.t, a.p, /*use_default=*/0,
+                         query_compute_units(), &chosen);
         if (st != FFA_OK) return st;
     }
-    st = validate_plan(chosen, precision, a.Dh, a.B * a.H, a.t, a.p);
+    st = validate_plan(chosen, planner_precision(precision), a.Dh, a.B * a.H, a.t, a.p);
     if (st != FFA_OK) return st;
     const size_t need = plan_workspace_bytes(chosen, a.B * a.H, a.Dh, a.Lmax);
     if (need > kStaticScratchBytes) return FFA_ERR_SCRATCH_LIMIT;

@@ -8,6 +8,21 @@
 namespace ffa {
 
 typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+
+// bfloat16 element (1-8-7), carried as its bit pattern like fp16 is carried as uint16_t.
+struct bf16_t {
+    uint16_t bits;
+};
+__device__ __forceinline__ float bf16_to_float(uint16_t b) {
+    return __builtin_bit_cast(float, (uint32_t)b << 16);
+}
+// Round-to-nearest-even; NaN stays NaN (quiet).
+__device__ __forceinline__ uint16_t float_to_bf16(float f) {
+    const uint32_t u = __builtin_bit_cast(uint32_t, f);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x40u);
+    return (uint16_t)((u + 0x7fffu + ((u >> 16) & 1u)) >> 16);
+}
 
 constexpr int kWave = 64;
 constexpr float kLog2e = 1.4426950408889634f;
@@ -57,6 +72,7 @@ __device__ __forceinline__ unsigned wave_sum_u32(unsigned x) {
 template <typename T> struct Elem;
 template <> struct Elem<uint16_t> { static constexpr int X = 8; };
 template <> struct Elem<float>    { static constexpr int X = 4; };
+template <> struct Elem<bf16_t>   { static constexpr int X = 8; };
 
 // 16-byte accesses to the KV caches carry the non-temporal hint (`nt`): every byte is used
 // once per step, and keeping the stream out of the caches' replacement order is worth 9-10 %
@@ -92,6 +108,14 @@ __device__ __forceinline__ float dot_chunk(const uint4& a, const uint4& b, float
     return acc;
 }
 
+__device__ __forceinline__ float dot_chunk(const uint4& a, const uint4& b, float acc, bf16_t) {
+    const bf16x2_t* x = reinterpret_cast<const bf16x2_t*>(&a);
+    const bf16x2_t* y = reinterpret_cast<const bf16x2_t*>(&b);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) acc = __builtin_amdgcn_fdot2_f32_bf16(x[i], y[i], acc, false);
+    return acc;
+}
+
 // acc[0..X) += p * chunk, fp32 accumulation.
 __device__ __forceinline__ void fma_chunk(float (&acc)[8], float p, const uint4& v, uint16_t) {
     const _Float16* h = reinterpret_cast<const _Float16*>(&v);
@@ -104,12 +128,22 @@ __device__ __forceinline__ void fma_chunk(float (&acc)[4], float p, const uint4&
     for (int i = 0; i < 4; ++i) acc[i] = fmaf(p, f[i], acc[i]);
 }
 
+__device__ __forceinline__ void fma_chunk(float (&acc)[8], float p, const uint4& v, bf16_t) {
+    const uint32_t* w = reinterpret_cast<const uint32_t*>(&v);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {   // a bf16 is the upper half of an fp32
+        acc[2 * i] = fmaf(p, __builtin_bit_cast(float, w[i] << 16), acc[2 * i]);
+        acc[2 * i + 1] = fmaf(p, __builtin_bit_cast(float, w[i] & 0xffff0000u), acc[2 * i + 1]);
+    }
+}
+
 // Final store of one output element.
 __device__ __forceinline__ void store_out(uint16_t* out, int idx, float v) {
     const _Float16 h = (_Float16)v;  // round-to-nearest-even
     out[idx] = __builtin_bit_cast(uint16_t, h);
 }
 __device__ __forceinline__ void store_out(float* out, int idx, float v) { out[idx] = v; }
+__device__ __forceinline__ void store_out(bf16_t* out, int idx, float v) { out[idx].bits = float_to_bf16(v); }
 
 // ---------------------------------------------------------------------------------------
 // The reference's pruning predicate.
@@ -128,6 +162,13 @@ __device__ __forceinline__ float round_prob(float x, uint16_t, float* key) {
 __device__ __forceinline__ float round_prob(float x, float, float* key) {
     *key = x;
     return x;
+}
+// bf16: the reference never enables its bf16 build, so there is no bit-pattern quirk to follow:
+// the probability rounded to bf16 is compared numerically, as the fp32 rule does.
+__device__ __forceinline__ float round_prob(float x, bf16_t, float* key) {
+    const float r = bf16_to_float(float_to_bf16(x));
+    *key = r;
+    return r;
 }
 
 }  // namespace ffa

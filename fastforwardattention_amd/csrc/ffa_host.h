@@ -15,6 +15,13 @@ constexpr int kMaxSplitWorkgroups = 16384;  // upper bound on workgroups of a sp
 constexpr int kMaxDynamicLdsBytes = 160 * 1024 - 20 * 1024;  // gfx950: 160 KiB LDS per CU, minus statics
                                                              // (16 KiB of survivor queues at 16 waves)
 
+// Bytes per element of a precision code (fp16 and bf16: 2, fp32: 4; 0 = unknown).
+inline int elem_bytes(int precision) {
+    return precision == FFA_PRECISION_F32 ? 4 : (precision == FFA_PRECISION_F16 || precision == FFA_PRECISION_BF16) ? 2 : 0;
+}
+// The planner and its table know two element sizes: bf16 plans like fp16.
+inline int planner_precision(int precision) { return precision == FFA_PRECISION_BF16 ? FFA_PRECISION_F16 : precision; }
+
 // Arguments of one decode step, after validation.
 struct DecodeArgs {
     int precision;
@@ -27,7 +34,15 @@ struct DecodeArgs {
     uint32_t* kept_count;
     uint8_t* skip_mask;
     void* stream;
+    // Bias and rotary embedding applied to the new token before the step (all optional).
+    const void *q_bias = nullptr, *k_bias = nullptr, *v_bias = nullptr;  // [H, Dh]
+    int rotary_dim = 0;
+    float rotary_base = 10000.f;
+    void* token_scratch = nullptr;  // 3 * B*H*Dh elements: the transformed q, k, v
+
+    bool transforms_token() const { return q_bias || k_bias || v_bias || rotary_dim > 0; }
 };
+
 
 // Carved-up workspace for a given plan.
 struct WorkspaceView {
@@ -41,6 +56,10 @@ struct WorkspaceView {
 inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 
 inline int num_tiles(int t) { return t / kTileKeys + 1; }  // keys 0..t inclusive
+
+// Scratch for the transformed new token (q, k, v), sized for the widest element; it sits behind
+// whatever the launch plan itself needs of the workspace.
+inline size_t token_scratch_bytes(int bh, int head_dim) { return align_up((size_t)3 * bh * head_dim * 4, 256); }
 
 // Dynamic LDS of the one-workgroup-per-(b,h) kernel: the larger of the score buffer and
 // the cross-wave merge buffer.

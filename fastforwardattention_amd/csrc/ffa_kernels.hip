@@ -1155,6 +1155,73 @@ __global__ void __launch_bounds__(256) ffa_init_cache_kernel(uint4* __restrict__
     }
 }
 
+// ---------------------------------------------------------------------------------------
+// New-token prologue of ffa_attention_ex: q += q_bias, k += k_bias, v += v_bias, then the
+// rotary embedding of q and k (attention.cu:856-882; the pair rotation and its angle are
+// decoder_masked_multihead_attention_utils.h:1137-1160).  One thread per pair of adjacent
+// elements of one (b,h).  Output: the three transformed tensors, [B,H,Dh] each, in the
+// workspace.
+struct TokenParams {
+    const void *q, *k, *v, *q_bias, *k_bias, *v_bias;
+    void *q_out, *k_out, *v_out;
+    const int* seq_lengths;
+    int H, Dh, t, right_or_no_padding, rotary_dim, n_pairs;
+    float rotary_base;
+};
+
+__device__ __forceinline__ double2 load_pair(const uint16_t* p) {
+    const half2_t h = *reinterpret_cast<const half2_t*>(p);
+    return make_double2((double)(float)h.x, (double)(float)h.y);
+}
+__device__ __forceinline__ double2 load_pair(const float* p) { return make_double2(p[0], p[1]); }
+__device__ __forceinline__ double2 load_pair(const bf16_t* p) {
+    return make_double2(bf16_to_float(p[0].bits), bf16_to_float(p[1].bits));
+}
+__device__ __forceinline__ void store_pair(uint16_t* p, float2 v) {
+    half2_t h = {(_Float16)v.x, (_Float16)v.y};
+    *reinterpret_cast<half2_t*>(p) = h;
+}
+__device__ __forceinline__ void store_pair(float* p, float2 v) { p[0] = v.x; p[1] = v.y; }
+__device__ __forceinline__ void store_pair(bf16_t* p, float2 v) {
+    p[0].bits = float_to_bf16(v.x);
+    p[1].bits = float_to_bf16(v.y);
+}
+
+// Arithmetic in fp64 (the angle pos / base^(2i/d) reaches hundreds of radians, where an fp32
+// angle is only good to 1e-5 and two math libraries no longer agree on its cosine), the result
+// rounded to fp32 and then once to T.  The reference does the same sums and products in fp32
+// (utils.h:1137-1156) after adding the bias in T (attention.cu:870-873).
+template <typename T>
+__global__ void __launch_bounds__(256) ffa_prepare_token_kernel(const TokenParams P) {
+    const int idx = blockIdx.x * 256 + threadIdx.x;
+    if (idx >= P.n_pairs) return;
+    const int half_dh = P.Dh >> 1;
+    const int bh = idx / half_dh, z = idx - bh * half_dh;  // elements 2z, 2z+1 of pair (b,h)
+    const int b = bh / P.H, h = bh - b * P.H;
+    const size_t e = (size_t)bh * P.Dh + 2 * z, eb = (size_t)h * P.Dh + 2 * z;
+    double2 q = load_pair(static_cast<const T*>(P.q) + e);
+    double2 k = load_pair(static_cast<const T*>(P.k) + e);
+    double2 v = load_pair(static_cast<const T*>(P.v) + e);
+    if (P.q_bias) { const double2 x = load_pair(static_cast<const T*>(P.q_bias) + eb); q.x += x.x; q.y += x.y; }
+    if (P.k_bias) { const double2 x = load_pair(static_cast<const T*>(P.k_bias) + eb); k.x += x.x; k.y += x.y; }
+    if (P.v_bias) { const double2 x = load_pair(static_cast<const T*>(P.v_bias) + eb); v.x += x.x; v.y += x.y; }
+    if (2 * z < P.rotary_dim) {
+        // Position of the new token among the sample's real tokens.
+        int pos = P.t;
+        if (P.seq_lengths != nullptr) {
+            const int sl = P.seq_lengths[b];
+            pos = P.right_or_no_padding ? min(max(sl, 0), P.t) : max(P.t - max(sl, 0), 0);
+        }
+        const double angle = (double)pos / pow((double)P.rotary_base, (double)(2 * z) / (double)P.rotary_dim);
+        const double c = cos(angle), s = sin(angle);
+        q = make_double2(c * q.x - s * q.y, c * q.y + s * q.x);
+        k = make_double2(c * k.x - s * k.y, c * k.y + s * k.x);
+    }
+    store_pair(static_cast<T*>(P.q_out) + e, make_float2((float)q.x, (float)q.y));
+    store_pair(static_cast<T*>(P.k_out) + e, make_float2((float)k.x, (float)k.y));
+    store_pair(static_cast<T*>(P.v_out) + e, make_float2((float)v.x, (float)v.y));
+}
+
 __global__ void ffa_fill_u32_kernel(unsigned int* p, size_t n, unsigned int v) {
     const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (i < n) p[i] = v;
@@ -1320,9 +1387,35 @@ static unsigned long long* g_trace = nullptr;
 extern "C" void ffa_debug_set_trace(void* p) { g_trace = static_cast<unsigned long long*>(p); }
 #endif
 
+template <typename T>
+static void launch_prepare_token(const DecodeArgs& a, hipStream_t st) {
+    TokenParams tp;
+    tp.q = a.q; tp.k = a.k; tp.v = a.v;
+    tp.q_bias = a.q_bias; tp.k_bias = a.k_bias; tp.v_bias = a.v_bias;
+    const size_t n = (size_t)a.B * a.H * a.Dh;
+    T* base = static_cast<T*>(a.token_scratch);
+    tp.q_out = base; tp.k_out = base + n; tp.v_out = base + 2 * n;
+    tp.seq_lengths = a.seq_lengths;
+    tp.H = a.H; tp.Dh = a.Dh; tp.t = a.t;
+    tp.right_or_no_padding = a.right_or_no_padding;
+    tp.rotary_dim = a.rotary_dim; tp.rotary_base = a.rotary_base;
+    tp.n_pairs = (int)(n / 2);
+    hipLaunchKernelGGL((ffa_prepare_token_kernel<T>), dim3((unsigned)((tp.n_pairs + 255) / 256)), dim3(256), 0, st, tp);
+}
+
 int launch_decode(const DecodeArgs& a, const ffa_launch_plan& plan, const WorkspaceView& ws) {
     DecodeParams P;
     P.q = a.q; P.k = a.k; P.v = a.v;
+    hipStream_t st = reinterpret_cast<hipStream_t>(a.stream);
+    if (a.transforms_token()) {
+        if (a.token_scratch == nullptr) return FFA_ERR_WORKSPACE;
+        if (a.precision == FFA_PRECISION_F16) launch_prepare_token<uint16_t>(a, st);
+        else if (a.precision == FFA_PRECISION_BF16) launch_prepare_token<bf16_t>(a, st);
+        else launch_prepare_token<float>(a, st);
+        const size_t n = (size_t)a.B * a.H * a.Dh * (a.precision == FFA_PRECISION_F32 ? 4 : 2);
+        const char* base = static_cast<const char*>(a.token_scratch);
+        P.q = base; P.k = base + n; P.v = base + 2 * n;
+    }
     P.k_cache = a.k_cache; P.v_cache = a.v_cache; P.out = a.out;
     P.seq_lengths = a.seq_lengths;
     P.ws_acc = ws.acc; P.ws_ml = ws.ml; P.ws_cnt = ws.cnt;
@@ -1339,8 +1432,8 @@ int launch_decode(const DecodeArgs& a, const ffa_launch_plan& plan, const Worksp
 #ifdef FFA_TRACE
     P.trace = g_trace;
 #endif
-    hipStream_t st = reinterpret_cast<hipStream_t>(a.stream);
     if (a.precision == FFA_PRECISION_F16) return dispatch_head_dim<uint16_t>(P, a.Dh, plan, st);
+    if (a.precision == FFA_PRECISION_BF16) return dispatch_head_dim<bf16_t>(P, a.Dh, plan, st);
     return dispatch_head_dim<float>(P, a.Dh, plan, st);
 }
 

@@ -33,9 +33,13 @@ void check_status(int st, const char* what) {
 int precision_of(const torch::Tensor& x) {
     if (x.scalar_type() == torch::kHalf) return FFA_PRECISION_F16;
     if (x.scalar_type() == torch::kFloat) return FFA_PRECISION_F32;
+    if (x.scalar_type() == torch::kBFloat16) return FFA_PRECISION_BF16;
     TORCH_CHECK(false, "ff_attention: unsupported tensor type ", x.scalar_type(),
-                " (float16 and float32 are supported)");
+                " (float16, bfloat16 and float32 are supported)");
 }
+
+// The planner knows two element sizes: bf16 plans like fp16.
+int plan_precision(int precision) { return precision == FFA_PRECISION_BF16 ? FFA_PRECISION_F16 : precision; }
 
 void* stream_of(const torch::Tensor& x) {
     return static_cast<void*>(c10::hip::getCurrentHIPStreamMasqueradingAsCUDA(x.device().index()).stream());
@@ -99,7 +103,7 @@ struct FastForwardAttn {
         v_cache = torch::empty({B, H, max_timesteps, Dh}, K.options());
         void* st = stream_of(K);
         int rc;
-        if (precision == FFA_PRECISION_F16)
+        if (precision != FFA_PRECISION_F32)  // fp16 and bf16 alike: cache construction moves 16-byte chunks
             rc = ffa_init_cache_f16((uint16_t*)k_cache.data_ptr(), (uint16_t*)v_cache.data_ptr(),
                                     (const uint16_t*)K.data_ptr(), (const uint16_t*)V.data_ptr(), B, L,
                                     max_timesteps, Dh, H, st);
@@ -138,6 +142,32 @@ struct FastForwardAttn {
 
     std::pair<torch::Tensor, torch::Tensor> get_cache() { return std::make_pair(k_cache, v_cache); }
 
+    // Not in the reference's Python surface: the step with the FasterTransformer features its host
+    // code switches off (attention.cu:1472-1483) -- q/k/v bias [H,Dh] and the rotary embedding of
+    // q and k over the first rotary_dim elements (GPT-J's pairing), applied to the new token
+    // before it is attended and appended.  seq_lengths = None, or int32 [B] first real keys of
+    // a left-padded batch; biases may be None.
+    torch::Tensor attention_ex(torch::Tensor q, torch::Tensor k, torch::Tensor v, torch::Tensor k_cache,
+                               torch::Tensor v_cache, float softmax_scale, int curr_timestep,
+                               c10::optional<torch::Tensor> seq_lengths, float prob_thresh, int rotary_dim,
+                               c10::optional<torch::Tensor> q_bias, c10::optional<torch::Tensor> k_bias,
+                               c10::optional<torch::Tensor> v_bias) {
+        const CacheDims d = dims_of(k_cache, v_cache);
+        torch::Tensor bias[3];
+        const c10::optional<torch::Tensor>* in[3] = {&q_bias, &k_bias, &v_bias};
+        ffa_token_transform tt = {nullptr, nullptr, nullptr, rotary_dim, 0.f};
+        const void** slot[3] = {&tt.q_bias, &tt.k_bias, &tt.v_bias};
+        for (int i = 0; i < 3; ++i) {
+            if (!in[i]->has_value()) continue;
+            bias[i] = token_input(in[i]->value(), k_cache, (int64_t)d.H * d.Dh, "bias");
+            *slot[i] = bias[i].data_ptr();
+        }
+        torch::Tensor sl;
+        if (seq_lengths.has_value()) sl = seq_lengths.value();
+        return run(q, k, v, k_cache, v_cache, softmax_scale, curr_timestep, seq_lengths.has_value() ? &sl : nullptr,
+                   prob_thresh, !seq_lengths.has_value(), nullptr, nullptr, &tt);
+    }
+
     // Not in the reference: the same step plus what pruning dropped.
     // Returns (out [B,H,Dh], kept_count int32 [B,H], skip_mask uint8 [B,H,Lmax]).
     std::tuple<torch::Tensor, torch::Tensor, torch::Tensor> attention_diag(
@@ -157,7 +187,7 @@ struct FastForwardAttn {
     std::vector<int> launch_plan(int curr_timestep, float prob_thresh) {
         const CacheDims d = dims_of(k_cache, v_cache);
         ffa_launch_plan plan;
-        check_status(ffa_plan_launch(precision_of(k_cache), d.B, d.H, d.Dh, curr_timestep, prob_thresh,
+        check_status(ffa_plan_launch(plan_precision(precision_of(k_cache)), d.B, d.H, d.Dh, curr_timestep, prob_thresh,
                                      ft_kernel_launch ? 1 : 0, 0, &plan),
                      "launch planning");
         return {plan.kind, plan.waves_per_wg, plan.threads_per_key, plan.keys_per_wave, plan.n_splits,
@@ -180,7 +210,7 @@ private:
     torch::Tensor run(const torch::Tensor& q_in, const torch::Tensor& k_in, const torch::Tensor& v_in,
                       torch::Tensor& kc, torch::Tensor& vc, float softmax_scale, int t,
                       const torch::Tensor* seq_lengths, float prob_thresh, bool right_or_no_padding,
-                      torch::Tensor* kept, torch::Tensor* mask) {
+                      torch::Tensor* kept, torch::Tensor* mask, const ffa_token_transform* transform = nullptr) {
         TORCH_CHECK(kc.is_cuda() && vc.is_cuda() && kc.device() == vc.device() &&
                         kc.scalar_type() == vc.scalar_type(),
                     "ff_attention: caches must be GPU tensors of one dtype on one device");
@@ -210,9 +240,18 @@ private:
         ffa_launch_plan plan;
         const bool diag = kept != nullptr || mask != nullptr;
         // The default launch keeps diagnostics at any length; the exact split kernel has none.
-        check_status(ffa_plan_launch(precision, d.B, d.H, d.Dh, t, prob_thresh,
+        check_status(ffa_plan_launch(plan_precision(precision), d.B, d.H, d.Dh, t, prob_thresh,
                                      (ft_kernel_launch || diag) ? 1 : 0, 0, &plan),
                      "launch planning");
+        if (transform != nullptr) {
+            TORCH_CHECK(!diag, "ff_attention: diagnostics and a token transform cannot be combined");
+            check_status(ffa_attention_ex(precision, d.B, d.H, d.Dh, d.Lmax, softmax_scale, t, q.data_ptr(),
+                                          k.data_ptr(), v.data_ptr(), kc.data_ptr(), vc.data_ptr(), out.data_ptr(),
+                                          sl_ptr, prob_thresh, &plan, right_or_no_padding ? 1 : 0, transform,
+                                          workspace.data_ptr(), (size_t)workspace.numel(), stream_of(kc)),
+                         "attention");
+            return out;
+        }
         const int rc = ffa_attention_diag(
             precision, d.B, d.H, d.Dh, d.Lmax, softmax_scale, t, q.data_ptr(), k.data_ptr(), v.data_ptr(),
             kc.data_ptr(), vc.data_ptr(), out.data_ptr(), sl_ptr, prob_thresh, &plan,
@@ -241,6 +280,8 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
              py::overload_cast<torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor,
                                float, int, torch::Tensor, float>(&FastForwardAttn::attention),
              "Attention forward, left-padded batch")
+        .def("attention_ex", &FastForwardAttn::attention_ex,
+             "Attention forward with q/k/v bias and rotary embedding of the new token")
         .def("attention_diag", &FastForwardAttn::attention_diag,
              "Attention forward plus (kept_count, skip_mask) of the pruning rule")
         .def("launch_plan", &FastForwardAttn::launch_plan, "Launch plan for (t, p)");

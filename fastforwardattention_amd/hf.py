@@ -15,6 +15,11 @@ Written against the installed transformers (5.x) instead of a patched copy of it
   the concatenated history.
 * models that dispatch through transformers' attention-function registry (OPT) select the
   registered function `"ffa"`; GPT-J, which calls its own `_attn`, gets that method wrapped.
+* GPT-J's rotary embedding of the new token's q and k, which the reference leaves to torch
+  ahead of the call (modeling_gptj.py:231-247), is taken over by the engine on decode steps
+  (`attention_ex(..., rotary_dim, ...)`: the FasterTransformer feature of attention.cu:874-882):
+  the layer's forward is wrapped and skips the torch-side sin/cos gather, split, rotate and
+  concatenate.  `enable(model, fused_rotary=False)` keeps the reference's arrangement.
 
     from fastforwardattention_amd import hf
     hf.enable(model)
@@ -148,6 +153,21 @@ class FFALayer(CacheLayerMixin):
         self._pending = False
         return out
 
+    def attend_rotary(self, query, key, value, scale: float, rotary_dim: int):
+        """One decode step on un-rotated q, k: [B,H,Dh] each -> [B,H,Dh].  The engine rotates q
+        and k at position t - first_key[b] (the sample's real tokens so far, which is what
+        transformers passes as position_ids for a left-padded batch) and appends."""
+        if not self._hooked:
+            raise RuntimeError("FFACache: the prompt pass did not go through the 'ffa' hook")
+        if self.t >= self.max_len:
+            raise RuntimeError(f"FFACache: cache full ({self.max_len} slots = prompt + max_new_tokens)")
+        dt = self.dtype
+        k_cache, v_cache = self.engine.get_cache()
+        out = self.engine.attention_ex(query.to(dt), key.to(dt), value.to(dt), k_cache, v_cache, float(scale), self.t,
+                                       self.first_key, self.prob_thresh, int(rotary_dim), None, None, None)
+        self.t += 1
+        return out
+
 
 class FFACache(Cache):
     """`past_key_values` object that keeps every layer's keys and values inside a
@@ -206,15 +226,38 @@ def _gptj_attn(self, query, key, value, attention_mask=None, *rest):
     return self._ffa_original_attn(query, key, value, attention_mask, *rest)
 
 
+def _gptj_forward(self, hidden_states, layer_past=None, attention_mask=None, position_ids=None, use_cache=False,
+                  output_attentions=False, **kwargs):
+    """Replacement for GPTJAttention.forward on one-token steps with an FFACache: projections,
+    then the engine (rotary embedding, append, attention), then the output projection.  Every
+    other call goes to the layer's own forward."""
+    layer = None
+    if isinstance(layer_past, FFACache) and self.layer_idx is not None and len(layer_past.layers) > self.layer_idx:
+        layer = layer_past.layers[self.layer_idx]
+    if (layer is None or layer.engine is None or hidden_states.shape[1] != 1 or output_attentions
+            or not hasattr(layer.engine, "attention_ex")):
+        return self._ffa_original_forward(hidden_states, layer_past, attention_mask, position_ids, use_cache,
+                                          output_attentions, **kwargs)
+    B, H, Dh = hidden_states.shape[0], self.num_attention_heads, self.head_dim
+    q = self.q_proj(hidden_states).view(B, H, Dh)
+    k = self.k_proj(hidden_states).view(B, H, Dh)
+    v = self.v_proj(hidden_states).view(B, H, Dh)
+    out = layer.attend_rotary(q, k, v, 1.0 / float(self.scale_attn), self.rotary_dim if self.rotary_dim is not None else Dh)
+    out = self.out_proj(out.reshape(B, 1, H * Dh).to(hidden_states.dtype))
+    return self.resid_dropout(out), None
+
+
 def register():
     """Make `"ffa"` known to transformers' attention and mask registries (idempotent)."""
     AttentionInterface.register(ATTN_NAME, ffa_attention_forward)
     AttentionMaskInterface.register(ATTN_NAME, eager_mask)
 
 
-def enable(model):
+def enable(model, fused_rotary=True):
     """Route `model`'s decode steps through FastForwardAttn.  Pass an `FFACache` as
-    `past_key_values` afterwards; with any other cache the model behaves as before."""
+    `past_key_values` afterwards; with any other cache the model behaves as before.
+    fused_rotary: GPT-J's rotary embedding of the new token runs inside the engine's call
+    instead of in torch (no effect on models without one)."""
     register()
     wrapped = 0
     for mod in model.modules():
@@ -222,6 +265,9 @@ def enable(model):
             if not hasattr(mod, "_ffa_original_attn"):
                 mod._ffa_original_attn = mod._attn
                 mod._attn = types.MethodType(_gptj_attn, mod)
+            if fused_rotary and not hasattr(mod, "_ffa_original_forward") and hasattr(mod, "rotary_dim"):
+                mod._ffa_original_forward = mod.forward
+                mod.forward = types.MethodType(_gptj_forward, mod)
             wrapped += 1
     if wrapped == 0:
         model._ffa_previous_attn = model.config._attn_implementation
@@ -235,6 +281,9 @@ def disable(model):
         if hasattr(mod, "_ffa_original_attn"):
             del mod.__dict__["_attn"]          # the class's own method shows through again
             del mod._ffa_original_attn
+        if hasattr(mod, "_ffa_original_forward"):
+            del mod.__dict__["forward"]
+            del mod._ffa_original_forward
     prev = getattr(model, "_ffa_previous_attn", None)
     if prev is not None:
         model.config._attn_implementation = prev

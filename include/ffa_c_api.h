@@ -46,14 +46,19 @@ typedef enum ffa_status {
     FFA_ERR_PROB_THRESH = 10,   /* p is negative or NaN                                      */
     FFA_ERR_LAUNCH = 11,        /* the HIP runtime refused the launch                        */
     FFA_ERR_NO_DEVICE = 12,     /* no usable gfx950 device / HIP runtime error               */
-    FFA_ERR_SCRATCH_LIMIT = 13  /* ffa_attention_static_scratch: the plan needs more scratch */
+    FFA_ERR_SCRATCH_LIMIT = 13, /* ffa_attention_static_scratch: the plan needs more scratch */
                                 /* than FFA_STATIC_SCRATCH_BYTES                             */
+    FFA_ERR_TRANSFORM = 14      /* rotary_embedding_dim odd, negative or > head_dim, or a    */
+                                /* bias pointer not 16-byte aligned                          */
 } ffa_status;
 
 /* precision codes: the same integers the reference passes to get_launch_params
  * (torch_ffa_api.cpp:174). */
 #define FFA_PRECISION_F16 16
 #define FFA_PRECISION_F32 32
+/* bfloat16 (1-8-7), accepted by ffa_attention_ex only.  The reference carries a bf16 build
+ * (ENABLE_BF16, decoder_masked_multihead_attention_utils.h:44-125) that it never enables. */
+#define FFA_PRECISION_BF16 0xBF16
 
 /* Launch kinds. */
 #define FFA_LAUNCH_WORKGROUP 0  /* one workgroup per (batch, head); scores staged in LDS;   */
@@ -115,7 +120,8 @@ int ffa_plan_launch_rules(int precision, int batch_size, int head_num, int head_
                           int compute_units, ffa_launch_plan* plan);
 
 /* Bytes of device workspace sufficient for ANY plan this library produces for the
- * given problem (arrival counters, split partials, two-pass scores). */
+ * given problem (arrival counters, split partials, two-pass scores, the transformed token
+ * of ffa_attention_ex). */
 size_t ffa_workspace_bytes(int batch_size, int head_num, int head_dim, int max_seq_len);
 
 /* Zero the arrival counters of a workspace of ffa_workspace_bytes() bytes (they sit at its
@@ -181,6 +187,40 @@ int ffa_attention_diag(int precision, int batch_size, int head_num, int head_dim
                        const int* seq_lengths, float prob_thresh, const ffa_launch_plan* plan,
                        int right_or_no_padding, void* workspace, size_t workspace_bytes,
                        uint32_t* kept_count, uint8_t* skip_mask, void* stream);
+
+/*
+ * The decode step with the FasterTransformer features that the reference's kernel carries but
+ * its host code switches off (attention.cu:1472-1483): q/k/v bias (attention.cu:856-873,
+ * :1157-1158, :1242), rotary position embedding of q and k (attention.cu:874-882;
+ * decoder_masked_multihead_attention_utils.h:1137-1160) and a bf16 element type.
+ *   precision  FFA_PRECISION_F16 | FFA_PRECISION_F32 | FFA_PRECISION_BF16 (bf16 caches are built
+ *              with ffa_init_cache_f16: cache construction only moves 16-byte chunks);
+ *   transform  NULL = none (then the call equals ffa_attention_f16 / _f32).  Otherwise, before
+ *              the step and in this order: q += q_bias, k += k_bias, v += v_bias (device
+ *              [H, Dh] arrays of the element type, each may be NULL); then, if
+ *              rotary_embedding_dim > 0 (even, <= head_dim), the pairs (2i, 2i+1) below that
+ *              dimension of q and k are rotated by pos / base^(2i / rotary_embedding_dim),
+ *              computed in fp32 and rounded once (GPT-J's convention).  pos is the number of
+ *              real tokens before the new one: t, or seq_lengths[b] with right padding, or
+ *              t - seq_lengths[b] with left padding (the reference rotates by t alone and so
+ *              supports no padded batch, attention.cu:879).  The transformed k and v are what
+ *              the caches receive.  It runs as one small kernel ahead of the decode kernel on
+ *              the same stream; its output lives in the workspace.
+ */
+typedef struct ffa_token_transform {
+    const void* q_bias;
+    const void* k_bias;
+    const void* v_bias;
+    int32_t rotary_embedding_dim; /* 0 = no rotary embedding                                   */
+    float rotary_base;            /* 10000 in the reference (utils.h:1139); <= 0 selects that  */
+} ffa_token_transform;
+
+int ffa_attention_ex(int precision, int batch_size, int head_num, int head_dim, int max_seq_len,
+                     float softmax_scale, int t, const void* q, const void* k, const void* v,
+                     void* k_cache, void* v_cache, void* out, const int* seq_lengths,
+                     float prob_thresh, const ffa_launch_plan* plan, int right_or_no_padding,
+                     const ffa_token_transform* transform, void* workspace, size_t workspace_bytes,
+                     void* stream);
 
 /*
  * The same step for callers that cannot allocate device memory (code under HIP graph

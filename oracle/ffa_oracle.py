@@ -15,6 +15,10 @@ citations are file:line under the reference checkout.
   half_from_ushort_rn   cuda_fp16.h __half(unsigned short) == __ushort2half_rn
   leq_f16_bits          attention.cu:466-469              __hle on converted bit patterns
   pruned_decode_step    attention.cu:1108-1126, :1184-1191, :1227-1256
+  token_transform       attention.cu:856-882, :1157-1158, :1242 (bias);
+                        decoder_masked_multihead_attention_utils.h:1137-1160 (rotary)
+  f32_to_bf16_bits / bf16_bits_to_f32   utils.h:44-125 (the bf16 build the reference never
+                        enables): round-to-nearest-even truncation of an fp32 to 16 bits
 
 Pinning status (what independent evidence fixes each function):
   attn_closed_form   pinned: brute-force Python loops, torch.softmax/bmm, fp64, and the
@@ -25,6 +29,12 @@ Pinning status (what independent evidence fixes each function):
                      pinned: known answers of IEEE round-to-nearest-even at 11 significant
                      bits (2049->2048, 2051->2052, 65520->inf) and exhaustive comparison
                      with numpy's own uint16->float16 cast over all 65536 patterns.
+  token_transform    pinned: the installed transformers' GPT-J apply_rotary_pos_emb /
+                     create_sinusoidal_positions on fp32 tensors (same pairs, signs and
+                     angles), a rotation's invariants (norm of every pair, position 0 is
+                     the identity, angles add), and the bias as plain addition.
+  bf16 conversions   pinned: torch's own float32 -> bfloat16 cast over random, tie, tiny,
+                     huge and special values; bf16 -> fp32 is a 16-bit shift.
   pruned_decode_step parity unpinned against the reference binary: no reference script
                      ever runs p>0 and the CUDA source cannot be built here.  It is pinned
                      only by invariants (p=0 and sub-resolution p reproduce the unpruned
@@ -162,9 +172,79 @@ def leq_f16_bits(a_bits, b_bits) -> np.ndarray:
     return half_from_ushort_rn(a_bits) <= half_from_ushort_rn(b_bits)
 
 
+# --------------------------------------------------------------------------- bf16, rounding to T
+def f32_to_bf16_bits(x) -> np.ndarray:
+    """fp32 -> bf16 bit pattern, round-to-nearest-even on the 16 dropped bits; NaN stays NaN."""
+    u = np.ascontiguousarray(x, dtype=np.float32).view(np.uint32).astype(np.uint64)
+    r = ((u + 0x7FFF + ((u >> 16) & 1)) >> 16).astype(np.uint16)
+    nan = (u & 0x7FFFFFFF) > 0x7F800000
+    return np.where(nan, ((u >> 16) | 0x40).astype(np.uint16), r)
+
+
+def bf16_bits_to_f32(b) -> np.ndarray:
+    return (np.asarray(b, dtype=np.uint16).astype(np.uint32) << 16).view(np.float32)
+
+
+def round_to(x, elem: str) -> np.ndarray:
+    """x rounded to the element type T ("f16", "bf16" or "f32"), returned as fp32 values."""
+    x = np.asarray(x, dtype=np.float32)
+    if elem == "f16":
+        return x.astype(np.float16).astype(np.float32)
+    if elem == "bf16":
+        return bf16_bits_to_f32(f32_to_bf16_bits(x))
+    assert elem == "f32"
+    return x
+
+
+# --------------------------------------------------------------------------- bias and rotary embedding
+def rotary_angles(pos, rotary_dim, base=10000.0) -> np.ndarray:
+    """angle[b, i] = pos[b] / base^(2i / rotary_dim), i < rotary_dim/2
+    (rotary_embedding_coefficient, utils.h:1137-1141), in float64."""
+    zid = np.arange(0, rotary_dim, 2, dtype=np.float64)
+    denom = np.power(np.float64(np.float32(base)), zid / np.float64(rotary_dim))
+    return np.asarray(pos, dtype=np.float64).reshape(-1, 1) / denom[None, :]
+
+
+def token_transform(q, k, v, elem, q_bias=None, k_bias=None, v_bias=None, rotary_dim=0, pos=None,
+                    base=10000.0):
+    """What the reference's kernel does to the new token before attending (disabled by its
+    host code, attention.cu:1472-1483): q += q_bias, k += k_bias (attention.cu:856-873),
+    v += v_bias (:1242); then for every pair (2i, 2i+1) with 2i < rotary_dim, q and k are
+    rotated: (x, y) -> (c x - s y, c y + s x), c, s = cos, sin of rotary_angles (:874-882;
+    utils.h:1143-1156).  The reference evaluates this in fp32 after adding the bias in T; here
+    (and in the kernel this checks) it is evaluated in float64 on the T-valued inputs and
+    rounded to fp32, then once to T: an fp32 angle of hundreds of radians is uncertain by 1e-5,
+    more than an ulp of the result, and could not be checked across two math libraries.
+    q, k, v: [B,H,Dh]; biases [H,Dh]; pos [B] = position of the new token of each sample.
+    Returns fp32 arrays holding T-representable values."""
+    q, k, v = (np.asarray(a, dtype=np.float32).astype(np.float64) for a in (q, k, v))
+    if q_bias is not None:
+        q = q + np.asarray(q_bias, dtype=np.float32).astype(np.float64)[None]
+    if k_bias is not None:
+        k = k + np.asarray(k_bias, dtype=np.float32).astype(np.float64)[None]
+    if v_bias is not None:
+        v = v + np.asarray(v_bias, dtype=np.float32).astype(np.float64)[None]
+    if rotary_dim > 0:
+        ang = rotary_angles(pos, rotary_dim, base)                     # [B, rotary_dim/2]
+        c, s = np.cos(ang)[:, None, :], np.sin(ang)[:, None, :]
+        for a in (q, k):
+            x, y = a[..., 0:rotary_dim:2].copy(), a[..., 1:rotary_dim:2].copy()
+            a[..., 0:rotary_dim:2] = c * x - s * y
+            a[..., 1:rotary_dim:2] = c * y + s * x
+    return tuple(round_to(a.astype(np.float32), elem) for a in (q, k, v))
+
+
+def rotary_positions(B, t, seq_lengths=None, right_or_no_padding=True) -> np.ndarray:
+    """Position of the new token among the sample's real tokens: the slot it is written to
+    minus the first unmasked key (t; seq_lengths[b] with right padding; t - seq_lengths[b]
+    with left padding).  The reference rotates by t alone (attention.cu:879)."""
+    tlen, first = _bounds(B, t, seq_lengths, right_or_no_padding)
+    return np.maximum(tlen - first, 0)
+
+
 # --------------------------------------------------------------------------- pruning rule
 def pruned_decode_step(q, k, v, k_cache, v_cache, scale, t, p, seq_lengths=None,
-                       right_or_no_padding=True):
+                       right_or_no_padding=True, elem=None):
     """One decode step with threshold-p pruning, transcribed from attention.cu.
 
     Per (b,h), with e_i = exp(s_i - max over unmasked s) (0 if masked, :1111-1116),
@@ -177,6 +257,10 @@ def pruned_decode_step(q, k, v, k_cache, v_cache, scale, t, p, seq_lengths=None,
     Scores s_i, the P.V products and their sum are carried in fp32 here (the reference
     carries them in T; this build's contract is fp32 accumulation), the result is
     returned in fp32 before the final rounding to T.
+
+    elem = "bf16" (caches passed as fp32 arrays of bf16 values): T-rounding to bf16 and a
+    numeric P_i <= thr; the reference has no bf16 behaviour to follow (ENABLE_BF16 is never
+    defined), this is the fp32 rule with bf16 rounding.
 
     Returns (out [B,H,Dh] float32, skipped [B,H,Lmax] bool, P [B,H,Lmax] float32,
     thr [B,H] float32).  Mutates the caches (append)."""
@@ -205,7 +289,10 @@ def pruned_decode_step(q, k, v, k_cache, v_cache, scale, t, p, seq_lengths=None,
         inv = (f32(1) / (S + EPS_SUM)).astype(f32)
         Pf = (e * inv).astype(f32)
         thrf = (f32(p) * inv).astype(f32)
-        if is_half:
+        if elem == "bf16":
+            Pv, thrv = round_to(Pf, "bf16"), round_to(thrf, "bf16")
+            skip = Pv <= thrv
+        elif is_half:
             Ph = Pf.astype(np.float16)
             thrh = thrf.astype(np.float16)
             skip = leq_f16_bits(Ph.view(np.uint16), thrh.view(np.uint16))

@@ -1,0 +1,291 @@
+"""GPU parity of ffa_attention_ex: the bf16 element type and the new-token transform (q/k/v bias,
+rotary embedding), through the C ABI, against the CPU oracle.
+
+Tolerances.  fp16 / fp32 outputs: 1e-3 / 1e-6 max-abs against the float64 closed form, as in the
+other parity tests.  bf16 outputs: one bf16 ulp of the closed form (|err| <= 2^-7 |want| + 1e-5;
+the kernel accumulates in fp32 and rounds once, so the error is a single rounding, at most half
+an ulp, plus the rare value that sits on a rounding boundary).  The transformed k and v that land
+in the caches: the oracle's values (both sides evaluate the rotation in fp64), at most one ulp
+apart on fewer than 1 % of the elements; bit for bit when only a bias is added."""
+import ctypes as C
+
+import numpy as np
+import pytest
+import torch
+
+from fastforwardattention_amd import capi
+from oracle import ffa_oracle as O
+from tests.ffa_testlib import ptr
+from tests.test_gpu_parity import _plans
+
+pytestmark = pytest.mark.gpu
+
+ELEMS = {"f16": (capi.FFA_PRECISION_F16, torch.float16), "bf16": (capi.FFA_PRECISION_BF16, torch.bfloat16),
+         "f32": (capi.FFA_PRECISION_F32, torch.float32)}
+
+
+def _say(*a):
+    print(*a, flush=True)
+
+
+def _to_dev(x, elem):
+    """fp32 numpy values (already representable in `elem`) -> device tensor of that type."""
+    return torch.from_numpy(np.ascontiguousarray(x, dtype=np.float32)).to("cuda:0").to(ELEMS[elem][1])
+
+
+def _bits(t):
+    """Device tensor -> numpy array of its raw element bits."""
+    if t.dtype == torch.float32:
+        return t.cpu().numpy().view(np.uint32)
+    return t.view(torch.int16).cpu().numpy().view(np.uint16)
+
+
+class ExSession:
+    """Caches + workspace for one problem in any of the three element types, driven through
+    ffa_init_cache_* and ffa_attention_ex.  K, V: fp32 numpy arrays of representable values."""
+
+    def __init__(self, K, V, max_len, elem):
+        self.lib = capi.load()
+        self.elem, (self.precision, tdt) = elem, ELEMS[elem]
+        B, H, L, Dh = K.shape
+        self.B, self.H, self.L, self.Dh, self.Lmax = B, H, L, Dh, max_len
+        x = 4 if elem == "f32" else 8
+        self.k_cache = torch.zeros(B, H, Dh // x, max_len, x, dtype=tdt, device="cuda:0")
+        self.v_cache = torch.zeros(B, H, max_len, Dh, dtype=tdt, device="cuda:0")
+        Kd, Vd = _to_dev(K, elem), _to_dev(V, elem)
+        init = self.lib.ffa_init_cache_f32 if elem == "f32" else self.lib.ffa_init_cache_f16   # 16-byte moves
+        capi.check(init(ptr(self.k_cache), ptr(self.v_cache), ptr(Kd), ptr(Vd), B, L, max_len, Dh, H, None),
+                   "ffa_init_cache")
+        n = self.lib.ffa_workspace_bytes(B, H, Dh, max_len)
+        self.ws = torch.empty(n, dtype=torch.uint8, device="cuda:0")
+        capi.check(self.lib.ffa_workspace_init(ptr(self.ws), n, None), "ffa_workspace_init")
+        torch.cuda.synchronize()
+
+    def step(self, q, k, v, scale, t, p=0.0, plan=None, seq_lengths=None, rnp=True, transform=None,
+             expect=capi.FFA_OK):
+        qd, kd, vd = (_to_dev(a, self.elem) for a in (q, k, v))
+        out = torch.full((self.B, self.H, self.Dh), float("nan"), dtype=ELEMS[self.elem][1], device="cuda:0")
+        sl = None if seq_lengths is None else torch.from_numpy(np.asarray(seq_lengths, np.int32)).to("cuda:0")
+        tt, keep = None, []
+        if transform is not None:
+            tt = capi.TokenTransform()
+            for name in ("q_bias", "k_bias", "v_bias"):
+                b = transform.get(name)
+                if b is not None:
+                    keep.append(_to_dev(b, self.elem))
+                    setattr(tt, name, keep[-1].data_ptr())
+            tt.rotary_embedding_dim = transform.get("rotary_dim", 0)
+            tt.rotary_base = transform.get("base", 0.0)
+        rc = self.lib.ffa_attention_ex(self.precision, self.B, self.H, self.Dh, self.Lmax, float(scale), int(t),
+                                       ptr(qd), ptr(kd), ptr(vd), ptr(self.k_cache), ptr(self.v_cache), ptr(out),
+                                       ptr(sl), float(p), C.byref(plan) if plan is not None else None, int(rnp),
+                                       C.byref(tt) if tt is not None else None, ptr(self.ws), self.ws.numel(), None)
+        assert rc == expect, capi.STATUS_NAMES.get(rc, rc)
+        torch.cuda.synchronize()
+        return None if rc != capi.FFA_OK else out.float().cpu().numpy()
+
+
+def _inputs(seed, B, H, L, Dh, elem, kv_scale=1.0):
+    rng = np.random.default_rng(seed)
+    r = lambda *s: O.round_to(rng.standard_normal(s) * kv_scale, elem)
+    return rng, r(B, H, L, Dh), r(B, H, L, Dh), r(B, H, Dh), r(B, H, Dh), r(B, H, Dh)
+
+
+def _pack(K, V, Lmax, elem):
+    """(k_cache, v_cache) as fp32 value arrays in the 8- or 4-element chunk layout of `elem`."""
+    dt = np.float32 if elem == "f32" else np.float16          # only the chunk width matters here
+    x = 16 // np.dtype(dt).itemsize
+    B, H, L, Dh = K.shape
+    kc = np.zeros((B, H, Dh // x, Lmax, x), np.float32)
+    kc[:, :, :, :L, :] = K.reshape(B, H, L, Dh // x, x).transpose(0, 1, 3, 2, 4)
+    vc = np.zeros((B, H, Lmax, Dh), np.float32)
+    vc[:, :, :L] = V
+    return kc, vc
+
+
+def _ulp(x, elem):
+    """One ulp of `elem` at |x| (fp32 arrays)."""
+    bits = {"f16": 10, "bf16": 7, "f32": 23}[elem]
+    tiny = {"f16": 2.0 ** -14, "bf16": 2.0 ** -126, "f32": 2.0 ** -126}[elem]
+    return 2.0 ** (np.floor(np.log2(np.maximum(np.abs(x), tiny))) - bits)
+
+
+def _out_tol(want, elem):
+    return {"f16": 1e-3, "f32": 1e-6}.get(elem, None) or (2.0 ** -7 * np.abs(want) + 1e-5)
+
+
+# ------------------------------------------------------------------ bf16, exact
+@pytest.mark.parametrize("Dh", [64, 80, 128, 256])
+@pytest.mark.parametrize("t", [0, 65, 777])
+def test_bf16_exact_step_all_plans(Dh, t):
+    B, H, elem = 2, 3, "bf16"
+    Lmax = t + 3
+    _, K, V, q, k, v = _inputs(5000 + Dh + t, B, H, t, Dh, elem)
+    scale = 1.0 / np.sqrt(Dh)
+    kc0, vc0 = _pack(K, V, Lmax, elem)
+    want = O.decode_step(q, k, v, kc0, vc0, scale, t, acc=np.float64)
+    for name, plan in _plans(16, B, H, Dh, t):
+        _say("bf16 exact", Dh, t, name)
+        sess = ExSession(K, V, Lmax, elem)
+        got = sess.step(q, k, v, scale, t, plan=plan)
+        assert (np.abs(got - want) <= _out_tol(want, elem)).all(), (name, float(np.abs(got - want).max()))
+        np.testing.assert_array_equal(_bits(sess.k_cache), O.f32_to_bf16_bits(kc0), err_msg=name)
+        np.testing.assert_array_equal(_bits(sess.v_cache), O.f32_to_bf16_bits(vc0), err_msg=name)
+
+
+def test_bf16_iterative_decode_and_padding():
+    """OPT-1.3b shape in miniature with bf16 caches: 12 appended tokens with the library's own plan,
+    then a left-padded and a right-padded step."""
+    B, H, Dh, L, steps, elem = 2, 32, 64, 1000, 12, "bf16"
+    rng, K, V, *_ = _inputs(77, B, H, L, Dh, elem, kv_scale=0.5)
+    sess = ExSession(K, V, L + steps, elem)
+    kc, vc = _pack(K, V, L + steps, elem)
+    for i in range(steps):
+        q, k, v = (O.round_to(rng.standard_normal((B, H, Dh)), elem) for _ in range(3))
+        got = sess.step(q, k, v, 0.125, L + i)
+        want = O.decode_step(q, k, v, kc, vc, 0.125, L + i, acc=np.float64)
+        assert (np.abs(got - want) <= _out_tol(want, elem)).all(), i
+    np.testing.assert_array_equal(_bits(sess.k_cache), O.f32_to_bf16_bits(kc))
+    np.testing.assert_array_equal(_bits(sess.v_cache), O.f32_to_bf16_bits(vc))
+    t = L + steps - 1
+    for sl, rnp in (([0, 400], False), ([t, 500], True)):
+        q, k, v = (O.round_to(rng.standard_normal((B, H, Dh)), elem) for _ in range(3))
+        got = sess.step(q, k, v, 0.125, t, seq_lengths=sl, rnp=rnp)
+        want = O.decode_step(q, k, v, kc, vc, 0.125, t, seq_lengths=np.array(sl), right_or_no_padding=rnp,
+                             acc=np.float64)
+        assert (np.abs(got - want) <= _out_tol(want, elem)).all(), (sl, rnp)
+
+
+@pytest.mark.parametrize("p", [1e-3, 1e-2])
+def test_bf16_pruned_step_matches_rule(p):
+    """Pruning with bf16 probabilities: the fp32 rule with T = bf16 rounding (the reference has no
+    bf16 behaviour of its own).  Skip decisions may differ only where the probability is within
+    one bf16 ulp of the threshold; the output equals the rule's for the GPU's own skip set."""
+    B, H, Dh, L, elem = 2, 3, 64, 900, "bf16"
+    rng, K, V, q, k, v = _inputs(31, B, H, L, Dh, elem)
+    qd = q / np.linalg.norm(q, axis=-1, keepdims=True)
+    for b in range(B):
+        for h in range(H):
+            pos = rng.choice(L, 16, replace=False)
+            K[b, h, pos] = O.round_to(4 * qd[b, h] + 0.1 * rng.standard_normal((16, Dh)), elem)
+    Lmax, scale = L + 1, 0.125
+    kc0, vc0 = _pack(K, V, Lmax, elem)
+    want, skip, P, thr = O.pruned_decode_step(q, k, v, kc0.copy(), vc0.copy(), scale, L, p, elem="bf16")
+    ntiles = L // 64 + 1
+    Vall = np.concatenate([V, v[:, :, None]], axis=2)
+    for plan in (capi.make_plan(capi.FFA_LAUNCH_WORKGROUP, 4, 1, ntiles), capi.make_plan(capi.FFA_LAUNCH_WORKGROUP, 16, 1, ntiles),
+                 capi.make_plan(capi.FFA_LAUNCH_TWO_PASS, 4, -(-ntiles // 2), 2), None):
+        _say("bf16 pruned", p, plan)
+        sess = ExSession(K, V, Lmax, elem)
+        kept = torch.zeros(B, H, dtype=torch.int32, device="cuda:0")
+        mask = torch.zeros(B, H, Lmax, dtype=torch.uint8, device="cuda:0")
+        out = torch.zeros(B, H, Dh, dtype=torch.bfloat16, device="cuda:0")
+        qd_, kd_, vd_ = (_to_dev(a, elem) for a in (q, k, v))
+        rc = sess.lib.ffa_attention_diag(sess.precision, B, H, Dh, Lmax, scale, L, ptr(qd_), ptr(kd_), ptr(vd_),
+                                         ptr(sess.k_cache), ptr(sess.v_cache), ptr(out), None, p,
+                                         C.byref(plan) if plan is not None else None, 1, ptr(sess.ws), sess.ws.numel(),
+                                         ptr(kept), ptr(mask), None)
+        assert rc == capi.FFA_OK, capi.STATUS_NAMES.get(rc, rc)
+        torch.cuda.synchronize()
+        gmask = mask.cpu().numpy().astype(bool)
+        near = np.abs(P - thr[:, :, None]) <= 2.0 ** -6 * np.abs(thr[:, :, None])
+        assert not ((gmask != skip) & ~near).any()
+        np.testing.assert_array_equal(kept.cpu().numpy(), L - gmask[:, :, :L].sum(-1))
+        w = np.where(gmask[:, :, :L + 1], 0, P[:, :, :L + 1])
+        want_g = np.einsum("bhn,bhnd->bhd", w, Vall)
+        got = out.float().cpu().numpy()
+        assert (np.abs(got - want_g) <= 2.0 ** -6 * np.abs(want_g) + 2e-3).all()
+    assert skip[:, :, :L].mean() > 0.01 if p >= 1e-2 else True
+
+
+# ------------------------------------------------------------------ bias and rotary embedding
+def _check_transform(elem, B, H, Dh, L, rd, bias, padding, seed, plan=None):
+    rng, K, V, q, k, v = _inputs(seed, B, H, L, Dh, elem)
+    biases = {n: O.round_to(rng.standard_normal((H, Dh)), elem) for n in ("q_bias", "k_bias", "v_bias")} if bias else {}
+    sl, rnp = None, True
+    if padding == "left":
+        sl, rnp = rng.integers(0, L // 2, B), False
+    elif padding == "right":
+        sl, rnp = rng.integers(L // 2, L + 1, B), True
+    Lmax, scale = L + 2, 1.0 / np.sqrt(Dh)
+    pos = O.rotary_positions(B, L, sl, rnp)
+    q2, k2, v2 = O.token_transform(q, k, v, elem, biases.get("q_bias"), biases.get("k_bias"), biases.get("v_bias"), rd, pos)
+    kc, vc = _pack(K, V, Lmax, elem)
+    want = O.decode_step(q2, k2, v2, kc, vc, scale, L, seq_lengths=sl, right_or_no_padding=rnp, acc=np.float64)
+    sess = ExSession(K, V, Lmax, elem)
+    got = sess.step(q, k, v, scale, L, plan=plan, seq_lengths=sl, rnp=rnp, transform=dict(biases, rotary_dim=rd))
+    # a q' or k' element on a rounding boundary may come out one ulp apart: a little slack for the scores
+    slack = {"f16": 3e-4, "bf16": 0.0, "f32": 1e-6}[elem] if rd else 0.0
+    tol = _out_tol(want, elem) * (2 if elem == "bf16" and rd else 1) + slack
+    assert (np.abs(got - want) <= tol).all(), float(np.abs(got - want).max())
+    # the caches received the transformed k, v at the slot of each sample
+    gk = sess.k_cache.float().cpu().numpy()
+    gv = sess.v_cache.float().cpu().numpy()
+    slot = np.full(B, L) if (sl is None or not rnp) else np.asarray(sl)
+    for b in range(B):
+        gkb = gk[b, :, :, slot[b], :].reshape(H, Dh)
+        if rd:
+            # both sides evaluate in fp64: equal except where the value sits on a rounding boundary
+            assert (np.abs(gkb - k2[b]) <= _ulp(k2[b], elem) * 1.01).all()
+            assert (gkb != k2[b]).mean() < 0.01
+            assert (gkb[:, rd:] == k2[b][:, rd:]).all()
+        else:
+            np.testing.assert_array_equal(gkb, k2[b])
+        np.testing.assert_array_equal(gv[b, :, slot[b]], v2[b])
+        np.testing.assert_array_equal(gk[b, :, :, :slot[b]], kc[b, :, :, :slot[b]])     # history untouched
+    return got
+
+
+@pytest.mark.parametrize("elem", ["f16", "bf16", "f32"])
+@pytest.mark.parametrize("Dh,rd", [(64, 32), (256, 64), (128, 128), (80, 16)])
+@pytest.mark.parametrize("padding", ["none", "left", "right"])
+def test_rotary_and_bias(elem, Dh, rd, padding):
+    _say("rotary+bias", elem, Dh, rd, padding)
+    _check_transform(elem, 3, 4, Dh, 300, rd, True, padding, 900 + Dh + rd)
+    _check_transform(elem, 2, 2, Dh, 130, rd, False, padding, 901 + Dh + rd)
+
+
+@pytest.mark.parametrize("elem", ["f16", "f32"])
+def test_bias_only_is_exact_and_every_plan_takes_the_transform(elem):
+    B, H, Dh, L = 2, 3, 64, 333
+    prec = 16 if elem == "f16" else 32
+    for name, plan in _plans(prec, B, H, Dh, L)[:12]:
+        _say("bias only", elem, name)
+        _check_transform(elem, B, H, Dh, L, 0, True, "none", 5, plan=plan)
+        _check_transform(elem, B, H, Dh, L, 32, True, "left", 6, plan=plan)
+
+
+def test_rotary_matches_transformers_gptj_end_to_end():
+    """One GPT-J-shaped step (16 heads x 256, rotary_dim 64) in fp32: q, k rotated by the installed
+    transformers' own apply_rotary_pos_emb, attention in fp64 torch -- against the fused call."""
+    gptj = pytest.importorskip("transformers.models.gptj.modeling_gptj")
+    B, H, Dh, L, rd = 2, 16, 256, 200, 64
+    _, K, V, q, k, v = _inputs(11, B, H, L, Dh, "f32")
+    emb = gptj.create_sinusoidal_positions(512, rd)
+    sin, cos = torch.split(emb[torch.full((B,), L)][:, None, :], rd // 2, dim=-1)
+    rot = lambda x: torch.cat([gptj.apply_rotary_pos_emb(torch.from_numpy(x)[:, None][..., :rd], sin, cos),
+                               torch.from_numpy(x)[:, None][..., rd:]], -1)[:, 0]
+    q2, k2 = rot(q).double(), rot(k).double()
+    Kall = torch.cat([torch.from_numpy(K).double(), k2[:, :, None]], 2)
+    Vall = torch.cat([torch.from_numpy(V).double(), torch.from_numpy(v).double()[:, :, None]], 2)
+    w = torch.softmax(torch.einsum("bhd,bhnd->bhn", q2, Kall) / 16.0, -1)
+    want = torch.einsum("bhn,bhnd->bhd", w, Vall).numpy()
+    got = ExSession(K, V, L + 1, "f32").step(q, k, v, 1 / 16.0, L, transform=dict(rotary_dim=rd))
+    assert np.abs(got - want).max() <= 1e-4      # transformers' fp32 angle at position 200 is good to 2e-5 rad
+
+
+def test_transform_argument_validation():
+    B, H, Dh, L = 1, 2, 64, 20
+    _, K, V, q, k, v = _inputs(3, B, H, L, Dh, "f16")
+    sess = ExSession(K, V, L + 1, "f16")
+    for rd in (-2, 3, 66):
+        sess.step(q, k, v, 0.125, L, transform=dict(rotary_dim=rd), expect=capi.FFA_ERR_TRANSFORM)
+    tiny = torch.empty(64, dtype=torch.uint8, device="cuda:0")
+    x = _to_dev(q, "f16")
+    tt = capi.TokenTransform(rotary_embedding_dim=32)
+    rc = sess.lib.ffa_attention_ex(16, B, H, Dh, L + 1, 0.125, L, ptr(x), ptr(x), ptr(x), ptr(sess.k_cache),
+                                   ptr(sess.v_cache), ptr(x), None, 0.0, None, 1, C.byref(tt), ptr(tiny), 64, None)
+    assert rc == capi.FFA_ERR_WORKSPACE          # no room for the transformed token
+    rc = sess.lib.ffa_attention_ex(12, B, H, Dh, L + 1, 0.125, L, ptr(x), ptr(x), ptr(x), ptr(sess.k_cache),
+                                   ptr(sess.v_cache), ptr(x), None, 0.0, None, 1, None, ptr(sess.ws), sess.ws.numel(), None)
+    assert rc == capi.FFA_ERR_DTYPE

@@ -38,6 +38,20 @@ class OracleEngine:
                             seq_lengths=None if seq_lens is None else seq_lens.numpy(), right_or_no_padding=False)
         return torch.from_numpy(out.astype(np.float32))
 
+    def attention_ex(self, q, k, v, k_cache, v_cache, scale, t, seq_lens, p, rotary_dim, q_bias, k_bias, v_bias):
+        """The fused call: the oracle's token transform (rotary embedding at the position
+        t - first_key[b]), then the step."""
+        assert q_bias is None and k_bias is None and v_bias is None
+        shape = (self.B, self.H, self.Dh)
+        sl = None if seq_lens is None else seq_lens.numpy()
+        pos = O.rotary_positions(self.B, t, sl, False)
+        q2, k2, v2 = O.token_transform(q.detach().numpy().reshape(shape), k.detach().numpy().reshape(shape),
+                                       v.detach().numpy().reshape(shape), "f32", rotary_dim=rotary_dim, pos=pos)
+        self.rotary_calls = getattr(self, "rotary_calls", []) + [(t, rotary_dim, pos.tolist())]
+        rest = (p,) if seq_lens is None else (seq_lens, p)
+        return self.attention(torch.from_numpy(q2), torch.from_numpy(k2), torch.from_numpy(v2), k_cache, v_cache,
+                              scale, t, *rest)
+
 
 def tiny_opt(dtype=torch.float32):
     cfg = transformers.OPTConfig(vocab_size=96, hidden_size=128, num_hidden_layers=2, ffn_dim=256,
@@ -80,13 +94,15 @@ def teacher_forced_logits(model, ids, mask, steps, cache):
     return torch.stack(logits), cache
 
 
-@pytest.mark.parametrize("family", ["opt", "gptj"])
+@pytest.mark.parametrize("family", ["opt", "gptj", "gptj_torch_rotary"])
 def test_hook_bookkeeping_against_plain_cache(family):
+    fused = family != "gptj_torch_rotary"
+    family = family.split("_")[0]
     model = tiny_opt() if family == "opt" else tiny_gptj()
     ids, mask = padded_batch()
     steps = 6
     want, _ = teacher_forced_logits(model, ids, mask, steps, None)
-    hf.enable(model)
+    hf.enable(model, fused_rotary=fused)
     cache = hf.FFACache(max_new_tokens=steps, engine=OracleEngine)
     got, cache = teacher_forced_logits(model, ids, mask, steps, cache)
     assert float((got - want).abs().max()) < 2e-4
@@ -98,6 +114,11 @@ def test_hook_bookkeeping_against_plain_cache(family):
         assert all(c[1] == [0, 4] for c in layer.engine.calls)                       # first real key per sample
         # OPT scales q before the call (scale 1); GPT-J passes 1/sqrt(Dh) (modeling_gptj.py:265)
         assert all(abs(c[2] - (1.0 if family == "opt" else Dh ** -0.5)) < 1e-7 for c in layer.engine.calls)
+        if family == "gptj" and fused:
+            # the engine rotated q and k itself: rotary_dim of the config, position = real tokens so far
+            assert layer.engine.rotary_calls == [(9 + i, 32, [9 + i, 5 + i]) for i in range(steps)]
+        else:
+            assert not hasattr(layer.engine, "rotary_calls")
     assert cache.get_seq_length() == 9 + steps
     # the cache is full now: one more token must be refused, not written out of bounds
     full = torch.cat([mask, torch.ones(2, steps + 1, dtype=mask.dtype)], 1)
@@ -147,15 +168,22 @@ def test_generate_with_ffa_cache_matches_plain_generate():
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("family,dtype,tol", [("opt", torch.float16, 3e-2), ("opt", torch.float32, 2e-4),
-                                               ("gptj", torch.float16, 3e-2), ("gptj", torch.float32, 2e-4)])
+                                               ("gptj", torch.float16, 3e-2), ("gptj", torch.float32, 2e-4),
+                                               ("gptj_torch_rotary", torch.float16, 3e-2),
+                                               ("gptj_torch_rotary", torch.float32, 2e-4),
+                                               ("opt", torch.bfloat16, 0.25), ("gptj", torch.bfloat16, 0.25)])
 def test_hook_with_hip_engine(family, dtype, tol):
-    """The real extension behind the cache, on the GPU, left-padded batch included."""
+    """The real extension behind the cache, on the GPU, left-padded batch included.  GPT-J runs
+    with the rotary embedding inside the engine's call and, as in the reference, in torch.
+    bfloat16 (8 significant bits) is held to a quarter of a logit unit."""
     print("hf hook", family, dtype, flush=True)
+    fused = family != "gptj_torch_rotary"
+    family = family.split("_")[0]
     model = (tiny_opt(dtype) if family == "opt" else tiny_gptj(dtype)).to("cuda:0")
     ids, mask = padded_batch("cuda:0")
     steps = 8
     want, _ = teacher_forced_logits(model, ids, mask, steps, None)
-    hf.enable(model)
+    hf.enable(model, fused_rotary=fused)
     for use_default in (False, True):
         got, cache = teacher_forced_logits(model, ids, mask, steps,
                                            hf.FFACache(max_new_tokens=steps, use_default_kernel_launch=use_default))

@@ -35,11 +35,11 @@ def test_every_declared_symbol_is_exported_and_bound(lib):
 def test_version_and_status_strings(lib):
     assert lib.ffa_api_version() == 1
     seen = set()
-    for code in range(0, 14):
+    for code in range(0, 15):
         s = capi.status_string(code)
         assert s and s != "unknown status"
         seen.add(s)
-    assert len(seen) == 14
+    assert len(seen) == 15
     assert capi.status_string(99) == "unknown status"
 
 
@@ -135,6 +135,28 @@ def test_static_scratch_entry_validates_before_any_launch(lib):
     many = capi.make_plan(capi.FFA_LAUNCH_SPLIT, 1, 64, 1)
     assert call(B=4, H=32, Dh=256, Lmax=4097, t=4095, plan=many) == capi.FFA_ERR_SCRATCH_LIMIT
     assert "scratch" in capi.status_string(capi.FFA_ERR_SCRATCH_LIMIT)
+
+
+def test_attention_ex_validates_before_any_launch(lib):
+    """ffa_attention_ex: element types, the token transform's fields and the room for the
+    transformed token are checked on the host."""
+    def call(precision=16, Dh=64, t=10, rotary=0, q_bias=None, ws=None, ws_bytes=0, plan=None, transform=True):
+        tt = capi.TokenTransform(q_bias=q_bias, rotary_embedding_dim=rotary) if transform else None
+        return lib.ffa_attention_ex(precision, 2, 4, Dh, 128, 0.125, t, P, P, P, P, P, P, None, 0.0,
+                                    C.byref(plan) if plan is not None else None, 1,
+                                    C.byref(tt) if tt is not None else None, ws, ws_bytes, None)
+    wg = capi.make_plan(capi.FFA_LAUNCH_WORKGROUP, 4, 1, 1)
+    assert call(precision=8, plan=wg) == capi.FFA_ERR_DTYPE
+    assert call(precision=17, plan=wg) == capi.FFA_ERR_DTYPE
+    for rd in (-1, 7, 66):
+        assert call(rotary=rd, plan=wg) == capi.FFA_ERR_TRANSFORM
+    assert call(rotary=32, q_bias=C.c_void_p(0x1008), plan=wg) == capi.FFA_ERR_TRANSFORM
+    # a transform needs the workspace even with a one-workgroup plan: 3 * B*H*Dh * 4 bytes
+    for prec in (16, 32, capi.FFA_PRECISION_BF16):
+        assert call(precision=prec, rotary=32, plan=wg) == capi.FFA_ERR_WORKSPACE
+        assert call(precision=prec, rotary=32, plan=wg, ws=P, ws_bytes=6143) == capi.FFA_ERR_WORKSPACE
+    assert "rotary" in capi.status_string(capi.FFA_ERR_TRANSFORM)
+    assert lib.ffa_workspace_bytes(2, 4, 64, 128) >= 6144
 
 
 def test_init_cache_argument_validation(lib):

@@ -278,3 +278,85 @@ def test_pruned_fp16_threshold_in_subnormal_range_is_integer_compare():
     np.testing.assert_array_equal(skip[0, 0, :L][clear], want[clear])
     assert clear.mean() > 0.99
     assert 0.02 * L < skip.sum() < 0.98 * L
+
+
+# --------------------------------------------------------------------------- bf16, bias, rotary embedding
+def test_bf16_conversion_matches_torch_cast():
+    """f32_to_bf16_bits against torch's own float32 -> bfloat16 cast (an independent
+    implementation): random values over the whole exponent range, exact ties (round to even),
+    denormals, infinities; NaN stays NaN.  bf16 -> f32 is exact."""
+    rng = np.random.default_rng(0)
+    x = np.concatenate([
+        rng.standard_normal(200000).astype(np.float32),
+        (rng.standard_normal(50000) * 10.0 ** rng.uniform(-40, 38, 50000)).astype(np.float32),
+        np.array([0.0, -0.0, 1.0, np.inf, -np.inf, 3.4e38, 1e-45, 1.17549435e-38], np.float32),
+        # ties: mantissa bits 0x8000 below an even / odd kept part
+        np.array([0x3F808000, 0x3F818000, 0x3F80FFFF, 0x3F810001, 0x7F7F8000, 0x00008000, 0x00018000],
+                 np.uint32).view(np.float32),
+    ])
+    got = O.f32_to_bf16_bits(x)
+    want = torch.from_numpy(x).to(torch.bfloat16).view(torch.int16).numpy().view(np.uint16)
+    np.testing.assert_array_equal(got, want)
+    assert got[np.flatnonzero(x.view(np.uint32) == 0x3F808000)[0]] == 0x3F80      # tie -> even (down)
+    assert got[np.flatnonzero(x.view(np.uint32) == 0x3F818000)[0]] == 0x3F82      # tie -> even (up)
+    assert np.isnan(O.bf16_bits_to_f32(O.f32_to_bf16_bits(np.array([np.nan], np.float32))))[0]
+    np.testing.assert_array_equal(O.bf16_bits_to_f32(got).view(np.uint32), got.astype(np.uint32) << 16)
+    np.testing.assert_array_equal(O.round_to(x[:1000], "f16"), x[:1000].astype(np.float16).astype(np.float32))
+
+
+def test_rotary_matches_transformers_gptj():
+    """token_transform's rotary embedding against the installed transformers' GPT-J functions on
+    fp32 tensors: same element pairs (2i, 2i+1), same signs, same angles pos / 10000^(2i/d),
+    elements beyond rotary_dim untouched."""
+    gptj = pytest.importorskip("transformers.models.gptj.modeling_gptj")
+    rng = np.random.default_rng(1)
+    for Dh, rd in [(64, 32), (256, 64), (64, 64), (128, 2)]:
+        B, H = 3, 2
+        q, k, v = (rng.standard_normal((B, H, Dh)).astype(np.float32) for _ in range(3))
+        emb = gptj.create_sinusoidal_positions(2048, rd)
+        # The reference divides pos by base^(2i/d), transformers multiplies by the reciprocal: the
+        # fp32 angles differ by an ulp or two, i.e. by up to 1.2e-4 rad at position 1500 and by
+        # 4e-6 rad below position 40; the rotated values differ by that times |x| (<= 4.5 here).
+        for pos, tol in ((np.array([0, 7, 39]), 2e-5), (np.array([0, 640, 1500]), 6e-4)):
+            sin, cos = torch.split(emb[torch.from_numpy(pos)][:, None, :], rd // 2, dim=-1)
+            def ref(x):
+                x = torch.from_numpy(x)[:, None]                               # [B, 1, H, Dh]
+                return torch.cat([gptj.apply_rotary_pos_emb(x[..., :rd], sin, cos), x[..., rd:]], -1)[:, 0].numpy()
+            gq, gk, gv = O.token_transform(q, k, v, "f32", rotary_dim=rd, pos=pos)
+            assert np.abs(gq - ref(q)).max() <= tol and np.abs(gk - ref(k)).max() <= tol
+        np.testing.assert_array_equal(gv, v)
+        np.testing.assert_array_equal(gq[..., rd:], q[..., rd:])
+        np.testing.assert_array_equal(gq[0], q[0])                          # position 0: identity
+
+
+def test_token_transform_invariants():
+    """Rotations keep the norm of every pair, compose additively in the position, and the bias is a
+    plain addition made before the rotation; results are values of the element type."""
+    rng = np.random.default_rng(2)
+    B, H, Dh, rd = 2, 3, 64, 48
+    q, k, v = (rng.standard_normal((B, H, Dh)).astype(np.float32) for _ in range(3))
+    qb, kb, vb = (rng.standard_normal((H, Dh)).astype(np.float32) for _ in range(3))
+    pos = np.array([3, 41])
+    gq, gk, gv = O.token_transform(q, k, v, "f32", qb, kb, vb, rd, pos)
+    np.testing.assert_allclose(gv, v + vb[None], rtol=0, atol=1e-7)
+    pn = lambda a: a[..., 0:rd:2] ** 2 + a[..., 1:rd:2] ** 2
+    np.testing.assert_allclose(pn(gq), pn(q + qb[None]), rtol=2e-6)
+    np.testing.assert_allclose(pn(gk), pn(k + kb[None]), rtol=2e-6)
+    np.testing.assert_array_equal(gk[..., rd:], (k + kb[None])[..., rd:])
+    # rotating by pos1 then pos2 (no bias) = rotating by pos1 + pos2, up to the fp32 angle rounding
+    a1, _, _ = O.token_transform(q, k, v, "f32", rotary_dim=rd, pos=np.array([3, 5]))
+    a2, _, _ = O.token_transform(a1, k, v, "f32", rotary_dim=rd, pos=np.array([4, 6]))
+    a3, _, _ = O.token_transform(q, k, v, "f32", rotary_dim=rd, pos=np.array([7, 11]))
+    np.testing.assert_allclose(a2, a3, atol=5e-6)
+    # known answer: pair (1, 0) at pair index 0 (angle = pos) becomes (cos pos, sin pos)
+    e = np.zeros((1, 1, 8), np.float32)
+    e[0, 0, 0] = 1
+    r, _, _ = O.token_transform(e, e, e, "f32", rotary_dim=8, pos=np.array([2]))
+    np.testing.assert_allclose(r[0, 0, :2], [np.cos(2.0), np.sin(2.0)], atol=1e-7)
+    for elem in ("f16", "bf16"):
+        h, _, _ = O.token_transform(q, k, v, elem, qb, kb, vb, rd, pos)
+        np.testing.assert_array_equal(h, O.round_to(h, elem))
+        assert np.abs(h - gq).max() <= (2 ** -10 if elem == "f16" else 2 ** -7) * np.abs(gq).max()
+    np.testing.assert_array_equal(O.rotary_positions(3, 50), [50, 50, 50])
+    np.testing.assert_array_equal(O.rotary_positions(3, 50, [10, 50, 0], True), [10, 50, 0])
+    np.testing.assert_array_equal(O.rotary_positions(3, 50, [10, 50, 60], False), [40, 0, 0])
