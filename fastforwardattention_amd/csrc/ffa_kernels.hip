@@ -64,37 +64,7 @@ struct DecodeParams {
     int n_whole;  // (b,h) pairs [0, n_whole) get one workgroup each; the rest are split
     int bh_total;
     int combine;  // FFA_COMBINE_*
-#ifdef FFA_TRACE
-    unsigned long long* trace;  // [wave slot][16] timestamps, profiling builds only
-#endif
 };
-
-// Phase timestamps for profiling builds (-DFFA_TRACE): lane 0 of every wave stores the
-// 100 MHz wall clock into slot `s` of its row.  Compiles to nothing otherwise.
-#ifdef FFA_TRACE
-#define FFA_TP_ENTRY()                                                                         \
-    const unsigned long long ffa_t_entry = wall_clock64();                                     \
-    unsigned long long* ffa_row = nullptr;                                                     \
-    if (P.trace) {                                                                             \
-        const unsigned w = __builtin_amdgcn_readfirstlane(                                     \
-            blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6));                              \
-        ffa_row = P.trace + (size_t)w * 16;                                                    \
-        if ((threadIdx.x & 63) == 0) {                                                         \
-            ffa_row[9] = ffa_t_entry;                                                          \
-            ffa_row[8] = (unsigned long long)__builtin_amdgcn_s_getreg((31 << 11) | 4) |       \
-                         ((unsigned long long)__builtin_amdgcn_s_getreg((31 << 11) | 20) << 32); \
-        }                                                                                      \
-    }
-// FFA_TRACE=2 keeps only the points that cost no registers in the hot loop (3 and later).
-#define FFA_TP(s)                                                            \
-    do {                                                                     \
-        if ((FFA_TRACE < 2 || (s) >= 3) && ffa_row && (threadIdx.x & 63) == 0) \
-            ffa_row[(s)] = wall_clock64();                                    \
-    } while (0)
-#else
-#define FFA_TP(s) do {} while (0)
-#define FFA_TP_ENTRY() do {} while (0)
-#endif
 
 // Per-(b) bounds, attention.cu:805-817.  tlen = slot of the new token = number of cached
 // keys; first = first unmasked key.  Values are clamped so that a bad seq_lengths entry
@@ -290,11 +260,6 @@ __device__ __forceinline__ void finish_piece(const DecodeParams& P, int bh, int 
     using G = Geo<T, DH>;
     constexpr int X = G::X, LPR = G::LPR, NCH = G::NCH;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-#ifdef FFA_TRACE
-    unsigned long long* ffa_row = nullptr;
-    if (P.trace) ffa_row = P.trace + (size_t)__builtin_amdgcn_readfirstlane(blockIdx.x * NW + wave) * 16;
-#endif
-    FFA_TP(3);
     // ---- merge inside the wave: the RPI row groups (lanes with equal lane % LPR) ----
 #pragma unroll
     for (int off = LPR; off < kWave; off <<= 1) {
@@ -361,14 +326,11 @@ __device__ __forceinline__ void finish_piece(const DecodeParams& P, int bh, int 
         publish(&ml[0], M);
         publish(&ml[1], L);
     }
-    FFA_TP(4);
     wait_published();
-    FFA_TP(5);
     unsigned prev = 0;
     if (lane == 0)
         prev = __hip_atomic_fetch_add(&P.ws_cnt[bh], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     prev = __builtin_amdgcn_readfirstlane(prev);
-    FFA_TP(6);
     if (prev != (unsigned)(n_splits * NPUB - 1)) return;
     // Compiler-only barrier: the loads of the merge below must stay behind the counter
     // read-modify-write (in hardware they are ordered by the branch on its returned value).
@@ -407,7 +369,6 @@ __device__ __forceinline__ void finish_piece(const DecodeParams& P, int bh, int 
         }
         store_out(out, d, Lg > 0.f ? o / Lg : 0.f);
     }
-    FFA_TP(7);
     // Ready for the next launch on this stream (kernel boundaries order this store).
     if (lane == 0) __hip_atomic_store(&P.ws_cnt[bh], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
@@ -426,8 +387,6 @@ __global__ void __launch_bounds__(NW * 64) ffa_decode_split_kernel(const DecodeP
     __shared__ uint4 s_q[G::Q_LDS ? NCH : 1];
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    FFA_TP_ENTRY();
-    FFA_TP(0);
 
     // Work mapping.  The first n_whole workgroups each own a whole (b,h) pair and finish with
     // an LDS merge only; the remaining pairs are cut into n_splits pieces whose partials are
@@ -520,7 +479,6 @@ __global__ void __launch_bounds__(NW * 64) ffa_decode_split_kernel(const DecodeP
                 s = dot_k_group<T, CG, G::Q_LDS>(kn, g, q_reg, s_q, s);
             }
         }
-        FFA_TP(1);
 
         const bool valid = key <= tlen && key >= first;
         const float m_new = fmaxf(m_run, wave_max(valid ? s * P.scale_log2e : -INFINITY));
@@ -538,8 +496,6 @@ __global__ void __launch_bounds__(NW * 64) ffa_decode_split_kernel(const DecodeP
 
 #pragma unroll
         for (int e = 0; e < X; ++e) acc[e] *= alpha;
-
-        FFA_TP(2);
         const float* pst = &s_p[wave][rg * NVL];
 #pragma unroll
         for (int g = 0; g < NVL / VG; ++g) {
@@ -1382,11 +1338,6 @@ static int dispatch_head_dim(const DecodeParams& P, int head_dim, const ffa_laun
     }
 }
 
-#ifdef FFA_TRACE
-static unsigned long long* g_trace = nullptr;
-extern "C" void ffa_debug_set_trace(void* p) { g_trace = static_cast<unsigned long long*>(p); }
-#endif
-
 template <typename T>
 static void launch_prepare_token(const DecodeArgs& a, hipStream_t st) {
     TokenParams tp;
@@ -1429,9 +1380,6 @@ int launch_decode(const DecodeArgs& a, const ffa_launch_plan& plan, const Worksp
     P.n_whole = plan.kind == FFA_LAUNCH_SPLIT ? plan.whole_heads : 0;
     P.bh_total = a.B * a.H;
     P.combine = plan.combine;
-#ifdef FFA_TRACE
-    P.trace = g_trace;
-#endif
     if (a.precision == FFA_PRECISION_F16) return dispatch_head_dim<uint16_t>(P, a.Dh, plan, st);
     if (a.precision == FFA_PRECISION_BF16) return dispatch_head_dim<bf16_t>(P, a.Dh, plan, st);
     return dispatch_head_dim<float>(P, a.Dh, plan, st);
