@@ -287,7 +287,7 @@ def parity_check(wl):
             "reference": "fp32 torch bmm/softmax/bmm on the GPU over the upcast inputs, every step"}
 
 
-def cpu_baseline(wl, budget_s=10.0, max_steps=8192):
+def cpu_baseline(wl, budget_s=12.0, max_steps=40000):
     """The reference's CPU path restated (oracle/torch_attn.py) on the host cores, on the same
     workload (one layer's cache): passes over the decode loop t = prompt .. prompt+gen-1 are
     repeated until about `budget_s` seconds of CPU work have been timed."""
