@@ -512,21 +512,31 @@ def run_init_cache_bench():
     return {"kernel": "ffa_init_cache_kernel (cache construction, fp16)", "results": res}
 
 
-def run_hf_end_to_end(B=10, prompt=1000, new_tokens=128):
-    """The reference's end-to-end setting in miniature (summarize.py: OPT with a left-padded batch,
-    greedy decoding): an OPT-1.3b-shaped model with random weights (nothing is downloaded), prompt
-    of `prompt` tokens, `new_tokens` decode steps; wall time per generated token with transformers'
-    own cache and attention against the FFACache hook.  Reported beside the kernel figures; the
-    projections and MLPs of the model dominate a decode step, the attention call is what changes."""
+def run_hf_end_to_end(family="opt", B=None, prompt=None, new_tokens=128):
+    """The reference's end-to-end setting in miniature (summarize.py: a left-padded batch, greedy
+    decoding): an OPT-1.3b-shaped or GPT-J-6B-shaped model with random weights (nothing is
+    downloaded), `new_tokens` decode steps; wall time per generated token with transformers' own
+    cache and attention against the FFACache hook (for GPT-J with the rotary embedding of the new
+    token inside the engine's call and, as the reference does it, in torch).  Reported beside the
+    kernel figures; the projections and MLPs of the model dominate a decode step, the attention
+    call is what changes."""
     import torch
     import transformers
     from fastforwardattention_amd import hf
-    cfg = transformers.OPTConfig(vocab_size=50272, hidden_size=2048, num_hidden_layers=24, ffn_dim=8192,
-                                 num_attention_heads=32, max_position_embeddings=2048, word_embed_proj_dim=2048,
-                                 dropout=0.0, attention_dropout=0.0)
+    if family == "opt":
+        B, prompt = B or 10, prompt or 1000
+        cfg = transformers.OPTConfig(vocab_size=50272, hidden_size=2048, num_hidden_layers=24, ffn_dim=8192,
+                                     num_attention_heads=32, max_position_embeddings=2048, word_embed_proj_dim=2048,
+                                     dropout=0.0, attention_dropout=0.0)
+        build, label = transformers.OPTForCausalLM, "OPT-1.3b-shaped"
+    else:
+        B, prompt = B or 8, prompt or 2000
+        cfg = transformers.GPTJConfig(vocab_size=50400, n_positions=4096, n_embd=4096, n_layer=28, n_head=16,
+                                      rotary_dim=64, resid_pdrop=0.0, embd_pdrop=0.0, attn_pdrop=0.0)
+        build, label = transformers.GPTJForCausalLM, "GPT-J-6B-shaped"
     torch.manual_seed(0)
     with torch.device("cuda:0"):
-        model = transformers.OPTForCausalLM(cfg).half().eval()
+        model = build(cfg).half().eval()
     g = torch.Generator(device="cuda:0").manual_seed(0)
     ids = torch.randint(4, 50000, (B, prompt), device="cuda:0", generator=g)
     mask = torch.ones_like(ids)
@@ -534,43 +544,36 @@ def run_hf_end_to_end(B=10, prompt=1000, new_tokens=128):
     kw = dict(attention_mask=mask, max_new_tokens=new_tokens, min_new_tokens=new_tokens, do_sample=False,
               pad_token_id=1)
 
-    def timed(**extra):
+    def per_token(run):
+        """ms per generated token, the prompt pass excluded: (n tokens) - (1 token)."""
         with torch.no_grad():
-            model.generate(ids, **{**kw, **extra, "max_new_tokens": 4, "min_new_tokens": 4})   # warm-up
-            torch.cuda.synchronize()
-            t0 = time.perf_counter()
-            model.generate(ids, **{**kw, **extra, "max_new_tokens": 1, "min_new_tokens": 1})   # prompt pass + 1 token
-            torch.cuda.synchronize()
-            t1 = time.perf_counter()
-            out = model.generate(ids, **{**kw, **extra})
-            torch.cuda.synchronize()
-            t2 = time.perf_counter()
-        return out, ((t2 - t1) - (t1 - t0)) * 1e3 / (new_tokens - 1)
-
-    res = {}
-    for impl in ("sdpa", "eager"):
-        model.config._attn_implementation = impl
-        ref_out, ms = timed()
-        res[f"transformers_{impl}_ms_per_token"] = round(ms, 3)
-    hf.enable(model)
-    outs = {}
-    for name, default in (("ffa_tuned", False), ("ffa_default_launch", True)):
-        with torch.no_grad():
-            # a cache object serves one generate() call: build a new one per call
-            def run(n):
-                return model.generate(ids, **{**kw, "max_new_tokens": n, "min_new_tokens": n},
-                                      past_key_values=hf.FFACache(max_new_tokens=n, use_default_kernel_launch=default))
             run(4)
             torch.cuda.synchronize()
             t0 = time.perf_counter(); run(1); torch.cuda.synchronize()
             t1 = time.perf_counter(); out = run(new_tokens); torch.cuda.synchronize()
             t2 = time.perf_counter()
-        res[f"{name}_ms_per_token"] = round(((t2 - t1) - (t1 - t0)) * 1e3 / (new_tokens - 1), 3)
-        outs[name] = out
-    hf.disable(model)
+        return out, ((t2 - t1) - (t1 - t0)) * 1e3 / (new_tokens - 1)
+
+    res, ref_out = {}, None
+    for impl in (("sdpa", "eager") if family == "opt" else ("eager",)):
+        model.config._attn_implementation = impl
+        ref_out, ms = per_token(lambda n: model.generate(ids, **{**kw, "max_new_tokens": n, "min_new_tokens": n}))
+        res[f"transformers_{impl}_ms_per_token"] = round(ms, 3)
+    outs = {}
+    variants = [("ffa_tuned", False, True), ("ffa_default_launch", True, True)]
+    if family != "opt":
+        variants.append(("ffa_tuned_rotary_in_torch", False, False))
+    for name, default, fused in variants:
+        hf.enable(model, fused_rotary=fused)
+        # a cache object serves one generate() call: build a new one per call
+        outs[name], ms = per_token(lambda n: model.generate(
+            ids, **{**kw, "max_new_tokens": n, "min_new_tokens": n},
+            past_key_values=hf.FFACache(max_new_tokens=n, use_default_kernel_launch=default)))
+        res[f"{name}_ms_per_token"] = round(ms, 3)
+        hf.disable(model)
     res["same_tokens_as_transformers_eager"] = bool(torch.equal(outs["ffa_tuned"], ref_out))
     res["matching_token_fraction"] = round(float((outs["ffa_tuned"] == ref_out).double().mean().item()), 6)
-    return {"workload": f"OPT-1.3b-shaped random model, fp16, B={B}, prompt {prompt} (odd samples left-padded by 37), "
+    return {"workload": f"{label} random model, fp16, B={B}, prompt {prompt} (odd samples left-padded by 37), "
                         f"{new_tokens} greedy tokens; per-token time excludes the prompt pass", **res}
 
 
@@ -886,8 +889,9 @@ def main():
     ap.add_argument("--plan", default=None, help="kind,waves,tiles_per_split[,combine[,whole_heads]] (kind: 0 workgroup, 1 split; combine: 0 fused, 1 kernel)")
     ap.add_argument("--legs", default="graph,capi,ext", help="comma list of graph,capi,ext")
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--hf-end-to-end", action="store_true",
-                    help="only: decode an OPT-1.3b-shaped random model with and without the FFACache hook")
+    ap.add_argument("--hf-end-to-end", nargs="?", const="opt", default=None, choices=["opt", "gptj"],
+                    help="only: decode an OPT-1.3b-shaped (default) or GPT-J-6B-shaped random model with and "
+                         "without the FFACache hook")
     ap.add_argument("--no-parity", action="store_true", help="skip the untimed every-step parity check")
     ap.add_argument("--no-suite", action="store_true",
                     help="leave out the short rows for the other BASELINE configurations")
@@ -932,7 +936,7 @@ def main():
         print(json.dumps(run_init_cache_bench()))
         return
     if args.hf_end_to_end:
-        print(json.dumps(run_hf_end_to_end()))
+        print(json.dumps(run_hf_end_to_end(args.hf_end_to_end)))
         return
 
     plan_override = tuple(int(x) for x in args.plan.split(",")) if args.plan else None
