@@ -523,6 +523,9 @@ def run_hf_end_to_end(family="opt", B=None, prompt=None, new_tokens=128):
     import torch
     import transformers
     from fastforwardattention_amd import hf
+    beams = 1
+    if family == "opt-beams":            # beam search: 2 prompts x 5 beams = the 10 rows of the headline batch
+        family, beams, B = "opt", 5, B or 2
     if family == "opt":
         B, prompt = B or 10, prompt or 1000
         cfg = transformers.OPTConfig(vocab_size=50272, hidden_size=2048, num_hidden_layers=24, ffn_dim=8192,
@@ -542,7 +545,9 @@ def run_hf_end_to_end(family="opt", B=None, prompt=None, new_tokens=128):
     mask = torch.ones_like(ids)
     mask[1::2, :37] = 0                      # every other sample is left-padded by 37 tokens
     kw = dict(attention_mask=mask, max_new_tokens=new_tokens, min_new_tokens=new_tokens, do_sample=False,
-              pad_token_id=1)
+              pad_token_id=1, eos_token_id=None)
+    if beams > 1:
+        kw.update(num_beams=beams, length_penalty=0.0)
 
     def per_token(run):
         """ms per generated token, the prompt pass excluded: (n tokens) - (1 token)."""
@@ -568,13 +573,14 @@ def run_hf_end_to_end(family="opt", B=None, prompt=None, new_tokens=128):
         # a cache object serves one generate() call: build a new one per call
         outs[name], ms = per_token(lambda n: model.generate(
             ids, **{**kw, "max_new_tokens": n, "min_new_tokens": n},
-            past_key_values=hf.FFACache(max_new_tokens=n, use_default_kernel_launch=default)))
+            past_key_values=hf.FFACache(max_new_tokens=n, use_default_kernel_launch=default, num_beams=beams)))
         res[f"{name}_ms_per_token"] = round(ms, 3)
         hf.disable(model)
     res["same_tokens_as_transformers_eager"] = bool(torch.equal(outs["ffa_tuned"], ref_out))
     res["matching_token_fraction"] = round(float((outs["ffa_tuned"] == ref_out).double().mean().item()), 6)
+    how = "greedy" if beams == 1 else f"beam-search (num_beams={beams}, {B * beams} cache rows)"
     return {"workload": f"{label} random model, fp16, B={B}, prompt {prompt} (odd samples left-padded by 37), "
-                        f"{new_tokens} greedy tokens; per-token time excludes the prompt pass", **res}
+                        f"{new_tokens} {how} tokens; per-token time excludes the prompt pass", **res}
 
 
 def measure_row(name, use_default=False, steps=32, eager=True):
@@ -889,9 +895,9 @@ def main():
     ap.add_argument("--plan", default=None, help="kind,waves,tiles_per_split[,combine[,whole_heads]] (kind: 0 workgroup, 1 split; combine: 0 fused, 1 kernel)")
     ap.add_argument("--legs", default="graph,capi,ext", help="comma list of graph,capi,ext")
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--hf-end-to-end", nargs="?", const="opt", default=None, choices=["opt", "gptj"],
-                    help="only: decode an OPT-1.3b-shaped (default) or GPT-J-6B-shaped random model with and "
-                         "without the FFACache hook")
+    ap.add_argument("--hf-end-to-end", nargs="?", const="opt", default=None, choices=["opt", "gptj", "opt-beams"],
+                    help="only: decode an OPT-1.3b-shaped (default; opt-beams: with beam search) or GPT-J-6B-shaped "
+                         "random model with and without the FFACache hook")
     ap.add_argument("--no-parity", action="store_true", help="skip the untimed every-step parity check")
     ap.add_argument("--no-suite", action="store_true",
                     help="leave out the short rows for the other BASELINE configurations")

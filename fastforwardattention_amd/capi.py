@@ -25,7 +25,7 @@ STATUS_NAMES = {
     0: "FFA_OK", 1: "FFA_ERR_NULL_POINTER", 2: "FFA_ERR_DTYPE", 3: "FFA_ERR_HEAD_DIM",
     4: "FFA_ERR_SHAPE", 5: "FFA_ERR_TIMESTEP", 6: "FFA_ERR_ALIGNMENT", 7: "FFA_ERR_WORKSPACE",
     8: "FFA_ERR_PLAN", 9: "FFA_ERR_TOO_LONG", 10: "FFA_ERR_PROB_THRESH", 11: "FFA_ERR_LAUNCH",
-    12: "FFA_ERR_NO_DEVICE", 13: "FFA_ERR_SCRATCH_LIMIT", 14: "FFA_ERR_TRANSFORM",
+    12: "FFA_ERR_NO_DEVICE", 13: "FFA_ERR_SCRATCH_LIMIT", 14: "FFA_ERR_TRANSFORM", 15: "FFA_ERR_BEAM",
 }
 globals().update({name: code for code, name in STATUS_NAMES.items()})   # FFA_OK, FFA_ERR_* as ints
 
@@ -54,9 +54,15 @@ class TokenTransform(C.Structure):
                 ("rotary_embedding_dim", C.c_int32), ("rotary_base", C.c_float)]
 
 
+class BeamIndirection(C.Structure):
+    """struct ffa_beam_indirection."""
+    _fields_ = [("cache_indir", C.c_void_p), ("beam_width", C.c_int32)]
+
+
 _vp, _i, _f, _sz = C.c_void_p, C.c_int, C.c_float, C.c_size_t
 _PLAN_P = C.POINTER(LaunchPlan)
 _TT_P = C.POINTER(TokenTransform)
+_BI_P = C.POINTER(BeamIndirection)
 
 # name -> (restype, argtypes); one entry per declaration in include/ffa_c_api.h
 SIGNATURES = {
@@ -76,7 +82,7 @@ SIGNATURES = {
     "ffa_attention_diag": (_i, [_i, _i, _i, _i, _i, _f, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _f,
                                 _PLAN_P, _i, _vp, _sz, _vp, _vp, _vp]),
     "ffa_attention_ex": (_i, [_i, _i, _i, _i, _i, _f, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _f, _PLAN_P, _i, _TT_P,
-                              _vp, _sz, _vp]),
+                              _BI_P, _vp, _sz, _vp]),
     "ffa_attention_static_scratch": (_i, [_i, _i, _i, _i, _i, _f, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _f,
                                           _PLAN_P, _i, _vp]),
 }

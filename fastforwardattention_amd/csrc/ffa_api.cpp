@@ -25,6 +25,12 @@ int validate_decode(const DecodeArgs& a) {
         return FFA_ERR_ALIGNMENT;
     if (a.rotary_dim < 0 || a.rotary_dim > a.Dh || (a.rotary_dim & 1)) return FFA_ERR_TRANSFORM;
     if (!aligned16(a.q_bias) || !aligned16(a.k_bias) || !aligned16(a.v_bias)) return FFA_ERR_TRANSFORM;
+    if (a.cache_indir != nullptr) {
+        if ((reinterpret_cast<uintptr_t>(a.cache_indir) & 3u) != 0) return FFA_ERR_BEAM;
+        if (a.beam_width < 1 || a.B % a.beam_width != 0) return FFA_ERR_BEAM;
+        // Rows of a group are numbered beam * H * Lmax + key in 32 bits.
+        if ((long long)a.beam_width * a.H * a.Lmax >= (1ll << 31)) return FFA_ERR_BEAM;
+    }
     return FFA_OK;
 }
 
@@ -45,11 +51,15 @@ int run_decode(const DecodeArgs& args, const ffa_launch_plan* user_plan, void* w
         st = plan_launch(plan_prec, a.B, a.H, a.Dh, a.t, a.p, /*use_default=*/0, cus, &plan);
         if (st == FFA_OK && diag && plan.kind == FFA_LAUNCH_SPLIT)
             st = plan_launch(plan_prec, a.B, a.H, a.Dh, a.t, 1.f, 0, cus, &plan);
+        // The kernels with several lanes per key read a sample's own caches only.
+        if (st == FFA_OK && a.cache_indir != nullptr && plan.threads_per_key > 1)
+            st = plan_launch_ex(plan_prec, a.B, a.H, a.Dh, a.t, a.p, 0, cus, /*use_table=*/0, &plan);
         if (st != FFA_OK) return st;
     }
     st = validate_plan(plan, plan_prec, a.Dh, a.B * a.H, a.t, a.p);
     if (st != FFA_OK) return st;
     if (diag && plan.kind == FFA_LAUNCH_SPLIT) return FFA_ERR_PLAN;
+    if (a.cache_indir != nullptr && plan.threads_per_key > 1) return FFA_ERR_PLAN;
 
     WorkspaceView ws = {nullptr, nullptr, nullptr, nullptr, 0};
     const int bh = a.B * a.H;
@@ -125,6 +135,7 @@ const char* ffa_status_string(int status) {
         case FFA_ERR_PROB_THRESH: return "prob_thresh must be a finite number >= 0";
         case FFA_ERR_LAUNCH: return "HIP kernel launch failed";
         case FFA_ERR_NO_DEVICE: return "no usable HIP device";
+        case FFA_ERR_BEAM: return "bad beam indirection: table NULL or not 4-byte aligned, beam_width < 1 or not a divisor of batch_size, or beam_width * head_num * max_seq_len >= 2^31";
         case FFA_ERR_TRANSFORM: return "bad token transform: rotary dimension must be even and within [0, head_dim], biases 16-byte aligned";
         case FFA_ERR_SCRATCH_LIMIT: return "the launch plan needs more scratch than the library's static 4 MiB array holds";
         default: return "unknown status";
@@ -215,8 +226,8 @@ int ffa_attention_ex(int precision, int batch_size, int head_num, int head_dim, 
                      float softmax_scale, int t, const void* q, const void* k, const void* v,
                      void* k_cache, void* v_cache, void* out, const int* seq_lengths,
                      float prob_thresh, const ffa_launch_plan* plan, int right_or_no_padding,
-                     const ffa_token_transform* transform, void* workspace, size_t workspace_bytes,
-                     void* stream) {
+                     const ffa_token_transform* transform, const ffa_beam_indirection* beams,
+                     void* workspace, size_t workspace_bytes, void* stream) {
     DecodeArgs a;
     a.precision = precision;
     a.B = batch_size; a.H = head_num; a.Dh = head_dim; a.Lmax = max_seq_len; a.t = t;
@@ -231,6 +242,11 @@ int ffa_attention_ex(int precision, int batch_size, int head_num, int head_dim, 
         a.q_bias = transform->q_bias; a.k_bias = transform->k_bias; a.v_bias = transform->v_bias;
         a.rotary_dim = transform->rotary_embedding_dim;
         a.rotary_base = transform->rotary_base > 0.f ? transform->rotary_base : 10000.f;
+    }
+    if (beams != nullptr) {
+        if (beams->cache_indir == nullptr) return FFA_ERR_BEAM;
+        a.cache_indir = beams->cache_indir;
+        a.beam_width = beams->beam_width;
     }
     return run_decode(a, plan, workspace, workspace_bytes);
 }

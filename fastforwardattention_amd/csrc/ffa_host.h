@@ -39,6 +39,9 @@ struct DecodeArgs {
     int rotary_dim = 0;
     float rotary_base = 10000.f;
     void* token_scratch = nullptr;  // 3 * B*H*Dh elements: the transformed q, k, v
+    // Beam-search indirection (optional): source beam of every cached key, [B, Lmax].
+    const int* cache_indir = nullptr;
+    int beam_width = 1;
 
     bool transforms_token() const { return q_bias || k_bias || v_bias || rotary_dim > 0; }
 };

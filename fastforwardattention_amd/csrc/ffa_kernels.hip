@@ -64,6 +64,8 @@ struct DecodeParams {
     int n_whole;  // (b,h) pairs [0, n_whole) get one workgroup each; the rest are split
     int bh_total;
     int combine;  // FFA_COMBINE_*
+    const int* cache_indir;  // [B, Lmax] source beam of every cached key, or nullptr
+    int beam_width;          // samples per beam group (>= 1)
 };
 
 // Per-(b) bounds, attention.cu:805-817.  tlen = slot of the new token = number of cached
@@ -102,6 +104,56 @@ __device__ __forceinline__ void new_token_store(const NewToken& n, char* kc_bh, 
         st16(vc_bh + ((size_t)tlen * NCH + lane) * 16, n.v);
     }
 }
+
+// Beam-search indirection (attention.cu:1003, :1024-1033, :1143, :1195-1202).  Sample b is beam
+// b % beam_width of group b / beam_width; its cached key i is read from the caches of the
+// group's beam cache_indir[b][i], while the new token is always appended to the sample's own
+// caches.  With BEAM = false every method folds to the sample's own caches at compile time.
+template <bool BEAM>
+struct BeamRows {
+    const int* idx = nullptr;  // this sample's row of cache_indir
+    int last = 0;              // beam_width - 1
+    size_t sample_bytes = 0;   // bytes between consecutive samples of a cache
+    char* k_group = nullptr;   // head h of the group's first beam
+    char* v_group = nullptr;
+
+    __device__ __forceinline__ BeamRows(const DecodeParams& P, int b, int bh, size_t head_bytes) {
+        if constexpr (BEAM) {
+            const int first_beam = b - b % P.beam_width;
+            const size_t off = ((size_t)first_beam * P.H + (bh - b * P.H)) * head_bytes;
+            idx = P.cache_indir + (size_t)b * P.Lmax;
+            last = P.beam_width - 1;
+            sample_bytes = (size_t)P.H * head_bytes;
+            k_group = reinterpret_cast<char*>(P.k_cache) + off;
+            v_group = reinterpret_cast<char*>(P.v_cache) + off;
+        } else {
+            k_group = reinterpret_cast<char*>(P.k_cache) + (size_t)bh * head_bytes;
+            v_group = reinterpret_cast<char*>(P.v_cache) + (size_t)bh * head_bytes;
+        }
+    }
+    // Source beam of `key` (callers pass one key per lane: a coalesced 4-byte load).  A table
+    // entry outside [0, beam_width) is clamped, so that it can never address memory outside the
+    // group; keys that are not in the cache yet give 0.
+    __device__ __forceinline__ int beam(int key, int tlen) const {
+        if constexpr (BEAM) return key < tlen ? min(max(idx[key], 0), last) : 0;
+        else return 0;
+    }
+    __device__ __forceinline__ const char* k_of(int beam) const {
+        if constexpr (BEAM) return k_group + (size_t)beam * sample_bytes;
+        else return k_group;
+    }
+    __device__ __forceinline__ const char* v_of(int beam) const {
+        if constexpr (BEAM) return v_group + (size_t)beam * sample_bytes;
+        else return v_group;
+    }
+    // Row number of key `key` of beam `beam` counted from v_group in V rows, -1 for the new
+    // token (key == tlen): what the survivor queue stores.
+    __device__ __forceinline__ int v_row(int beam, int key, int tlen, int rows_per_sample) const {
+        if (key >= tlen) return -1;
+        if constexpr (BEAM) return beam * rows_per_sample + key;
+        else return key;
+    }
+};
 
 // ---------------------------------------------------------------------------------------
 // One 64-key tile of q.K^T for the calling wave.  Lane l owns key tile*64+l; keys beyond
@@ -185,7 +237,8 @@ __device__ __forceinline__ void wait_published() { asm volatile("s_waitcnt vmcnt
 // nor instructions, so the keys that survive are compacted, per wave, into an LDS queue of
 // two 64-entry blocks (weight + cache row each); a block is consumed as soon as it is full,
 // by the same V mapping as an ordinary tile: every lane active, every load a surviving row.
-// Entry n of the stream sits in block (n >> 6) & 1 at stage_slot(n & 63).
+// Entry n of the stream sits in block (n >> 6) & 1 at stage_slot(n & 63).  A cache row is a
+// V row number counted from `v_base` (BeamRows::v_row), -1 standing for the new token.
 struct SurvivorQueue {
     float* w;          // this wave's 128 weights
     int* row;          // this wave's 128 cache rows
@@ -195,8 +248,7 @@ struct SurvivorQueue {
 // P.V over one queue block holding `count` valid entries (64 unless it is the last one).
 template <typename T, int DH>
 __device__ __forceinline__ void pv_queue_block(float (&acc)[Elem<T>::X], const SurvivorQueue& q, int block,
-                                               int count, const char* vc_bh, const char* vnew, int tlen,
-                                               int lane) {
+                                               int count, const char* v_base, const char* vnew, int lane) {
     using G = Geo<T, DH>;
     constexpr int NCH = G::NCH, LPR = G::LPR, RPI = G::RPI, NVL = G::NVL, VG = G::VG;
     const int rg = lane / LPR, dch = min(lane % LPR, NCH - 1);
@@ -211,19 +263,19 @@ __device__ __forceinline__ void pv_queue_block(float (&acc)[Elem<T>::X], const S
             // Loads are unconditional (a load under a branch is waited for at the join, one
             // round trip per row): entries past `count` re-read the new token with weight 0.
             const int n = (g * VG + j) * RPI + rg;  // entry number inside the block
-            const int r = n < count ? pr[g * VG + j] : tlen;
+            const int r = n < count ? pr[g * VG + j] : -1;
             pj[j] = n < count ? pw[g * VG + j] : 0.f;
-            vv[j] = ld16(r < tlen ? vc_bh + ((size_t)r * NCH + dch) * 16 : vnew + dch * 16);
+            vv[j] = ld16(r >= 0 ? v_base + ((size_t)r * NCH + dch) * 16 : vnew + dch * 16);
         }
 #pragma unroll
         for (int j = 0; j < VG; ++j) fma_chunk(acc, pj[j], vv[j], T{});
     }
 }
 
-// Push this lane's key if it survives; consumes a block when one fills up.
+// Push this lane's key (cache row `row`) if it survives; consumes a block when one fills up.
 template <typename T, int DH>
 __device__ __forceinline__ void queue_push(float (&acc)[Elem<T>::X], SurvivorQueue& q, bool keep, float weight,
-                                           int key, const char* vc_bh, const char* vnew, int tlen, int lane) {
+                                           int row, const char* v_base, const char* vnew, int lane) {
     using G = Geo<T, DH>;
     const unsigned long long mask = __builtin_amdgcn_ballot_w64(keep);
     const unsigned before =
@@ -232,20 +284,20 @@ __device__ __forceinline__ void queue_push(float (&acc)[Elem<T>::X], SurvivorQue
         const unsigned n = q.total + before;
         const int slot = ((n >> 6) & 1) * kWave + stage_slot<G::NVL, G::RPI>(n & 63);
         q.w[slot] = weight;
-        q.row[slot] = key;
+        q.row[slot] = row;
     }
     const unsigned after = q.total + (unsigned)__builtin_popcountll(mask);
     __builtin_amdgcn_wave_barrier();
     if ((after >> 6) != (q.total >> 6))  // wave-uniform: a block has just been completed
-        pv_queue_block<T, DH>(acc, q, (q.total >> 6) & 1, kWave, vc_bh, vnew, tlen, lane);
+        pv_queue_block<T, DH>(acc, q, (q.total >> 6) & 1, kWave, v_base, vnew, lane);
     q.total = after;
     __builtin_amdgcn_wave_barrier();
 }
 
 template <typename T, int DH>
-__device__ __forceinline__ void queue_drain(float (&acc)[Elem<T>::X], SurvivorQueue& q, const char* vc_bh,
-                                            const char* vnew, int tlen, int lane) {
-    if (q.total & 63) pv_queue_block<T, DH>(acc, q, (q.total >> 6) & 1, q.total & 63, vc_bh, vnew, tlen, lane);
+__device__ __forceinline__ void queue_drain(float (&acc)[Elem<T>::X], SurvivorQueue& q, const char* v_base,
+                                            const char* vnew, int lane) {
+    if (q.total & 63) pv_queue_block<T, DH>(acc, q, (q.total >> 6) & 1, q.total & 63, v_base, vnew, lane);
 }
 
 // ---------------------------------------------------------------------------------------
@@ -375,7 +427,7 @@ __device__ __forceinline__ void finish_piece(const DecodeParams& P, int bh, int 
 
 // ---------------------------------------------------------------------------------------
 // Sequence-split exact decode (p == 0).
-template <typename T, int DH, int NW>
+template <typename T, int DH, int NW, bool BEAM>
 __global__ void __launch_bounds__(NW * 64) ffa_decode_split_kernel(const DecodeParams P) {
     using G = Geo<T, DH>;
     constexpr int X = G::X, NCH = G::NCH, LPR = G::LPR, RPI = G::RPI, NVL = G::NVL;
@@ -416,6 +468,8 @@ __global__ void __launch_bounds__(NW * 64) ffa_decode_split_kernel(const DecodeP
     const uint4* qg = reinterpret_cast<const uint4*>(reinterpret_cast<const char*>(P.q) +
                                                      (size_t)bh * DH * sizeof(T));
 
+    const BeamRows<BEAM> beams(P, b, bh, head_bytes);
+
     uint4 q_reg[G::QREG];
     if constexpr (G::Q_LDS) {
         if (tid < NCH) s_q[tid] = qg[tid];
@@ -441,12 +495,16 @@ __global__ void __launch_bounds__(NW * 64) ffa_decode_split_kernel(const DecodeP
 #pragma unroll
     for (int e = 0; e < X; ++e) acc[e] = 0.f;
 
-    // V rows of load group g for this lane: rows tile*64 + (g*VG+j)*RPI + rg, j < VG.
-    auto load_v_group = [&](uint4 (&vv)[VG], int tile, int g) {
+    // V rows of load group g for this lane: rows tile*64 + (g*VG+j)*RPI + rg, j < VG.  `src` is
+    // the source beam of this lane's key of the tile; a row's beam sits in the lane of that key.
+    auto load_v_group = [&](uint4 (&vv)[VG], int tile, int g, int src) {
 #pragma unroll
         for (int j = 0; j < VG; ++j) {
-            const int row = min(tile * kWave + (g * VG + j) * RPI + rg, tlen);
-            const char* vp = row < tlen ? vc_bh + ((size_t)row * NCH + dch) * 16 : vnew + dch * 16;
+            const int in_tile = (g * VG + j) * RPI + rg;
+            const int row = min(tile * kWave + in_tile, tlen);
+            const char* vb = vc_bh;
+            if constexpr (BEAM) vb = beams.v_of(__shfl(src, in_tile));
+            const char* vp = row < tlen ? vb + ((size_t)row * NCH + dch) * 16 : vnew + dch * 16;
             vv[j] = ld16(vp);
         }
     };
@@ -455,22 +513,22 @@ __global__ void __launch_bounds__(NW * 64) ffa_decode_split_kernel(const DecodeP
 
     // First load groups of one tile: CG chunks of K (lane = key) and VG chunks of V
     // (lane = row group x d-chunk).  V does not depend on the scores, so both go out together.
-    auto load_tile = [&](uint4 (&kv)[CG], uint4 (&vv)[VG], int tile) {
+    auto load_tile = [&](uint4 (&kv)[CG], uint4 (&vv)[VG], int tile, int src) {
         const int key = tile * kWave + lane;
         const bool cached = key < tlen;
-        const char* kp = cached ? kc_bh + (size_t)key * 16 : knew;
+        const char* kp = cached ? beams.k_of(src) + (size_t)key * 16 : knew;
         const size_t kstr = cached ? (size_t)P.Lmax * 16 : 16;
         load_k_group<CG>(kv, kp, kstr, 0);
-        load_v_group(vv, tile, 0);
+        load_v_group(vv, tile, 0, src);
     };
 
     // Scores, online softmax and P.V of one tile whose first load groups are in kv / vv.
-    auto compute_tile = [&](uint4 (&kv)[CG], uint4 (&vv)[VG], int tile) {
+    auto compute_tile = [&](uint4 (&kv)[CG], uint4 (&vv)[VG], int tile, int src) {
         const int key = tile * kWave + lane;
         float s = dot_k_group<T, CG, G::Q_LDS>(kv, 0, q_reg, s_q, 0.f);
         if constexpr (NCH > CG) {
             const bool cached = key < tlen;
-            const char* kp = cached ? kc_bh + (size_t)key * 16 : knew;
+            const char* kp = cached ? beams.k_of(src) + (size_t)key * 16 : knew;
             const size_t kstr = cached ? (size_t)P.Lmax * 16 : 16;
 #pragma unroll 2
             for (int g = 1; g < NCH / CG; ++g) {
@@ -500,7 +558,7 @@ __global__ void __launch_bounds__(NW * 64) ffa_decode_split_kernel(const DecodeP
 #pragma unroll
         for (int g = 0; g < NVL / VG; ++g) {
             uint4 vn[VG];
-            if (g + 1 < NVL / VG) load_v_group(vn, tile, g + 1);
+            if (g + 1 < NVL / VG) load_v_group(vn, tile, g + 1, src);
 #pragma unroll
             for (int j = 0; j < VG; ++j) fma_chunk(acc, pst[g * VG + j], vv[j], T{});
             if (g + 1 < NVL / VG) {
@@ -512,12 +570,17 @@ __global__ void __launch_bounds__(NW * 64) ffa_decode_split_kernel(const DecodeP
     };
 
     // The scheduling barriers keep the compiler from sinking loads next to their uses to
-    // save registers, which would serialise the round trips.
+    // save registers, which would serialise the round trips.  With beam indirection the
+    // source beams of a tile are fetched one tile ahead, so that their round trip does not sit
+    // in front of the tile's own loads.
+    int src_next = beams.beam((tile_lo + wave) * kWave + lane, tlen);
     for (int tile = tile_lo + wave; tile < tile_hi; tile += NW) {
+        const int src = src_next;
+        if constexpr (BEAM) src_next = beams.beam((tile + NW) * kWave + lane, tile + NW < tile_hi ? tlen : 0);
         uint4 kv[CG], vv[VG];
-        load_tile(kv, vv, tile);
+        load_tile(kv, vv, tile, src);
         __builtin_amdgcn_sched_barrier(0);
-        compute_tile(kv, vv, tile);
+        compute_tile(kv, vv, tile, src);
     }
     if (appends) new_token_store<NCH>(new_tok, kc_bh, vc_bh, tlen, P.Lmax, lane);
 
@@ -660,7 +723,7 @@ __global__ void __launch_bounds__(64) ffa_merge_splits_kernel(const DecodeParams
 // ---------------------------------------------------------------------------------------
 // One workgroup per (b,h): exact (p == 0) or pruned (p > 0) decode with LDS-staged scores.
 // Dynamic LDS: max(ntiles*64 scores, NW*64*X merge floats) * 4 bytes.
-template <typename T, int DH, int NW>
+template <typename T, int DH, int NW, bool BEAM>
 __global__ void __launch_bounds__(NW * 64) ffa_decode_wg_kernel(const DecodeParams P) {
     using G = Geo<T, DH>;
     constexpr int X = G::X, NCH = G::NCH, LPR = G::LPR, RPI = G::RPI, NVL = G::NVL, VG = G::VG;
@@ -698,6 +761,9 @@ __global__ void __launch_bounds__(NW * 64) ffa_decode_wg_kernel(const DecodePara
         for (int c = 0; c < NCH; ++c) q_reg[c] = qg[c];
     }
 
+    const BeamRows<BEAM> beams(P, b, bh, head_bytes);
+    const int rows_per_sample = P.H * P.Lmax;
+
     const int ntiles = tlen / kWave + 1;
     const int tile_lo = min(first / kWave, ntiles);  // tiles below are fully masked
     const bool pruned = P.p > 0.f;
@@ -709,7 +775,7 @@ __global__ void __launch_bounds__(NW * 64) ffa_decode_wg_kernel(const DecodePara
     float mx = -INFINITY;
     for (int tile = tile_lo + wave; tile < ntiles; tile += NW) {
         const int key = tile * kWave + lane;
-        float s = tile_qk<T, NCH, G::Q_LDS>(kc_bh, knew, key, tlen, P.Lmax, q_reg, s_q);
+        float s = tile_qk<T, NCH, G::Q_LDS>(beams.k_of(beams.beam(key, tlen)), knew, key, tlen, P.Lmax, q_reg, s_q);
         const bool valid = key <= tlen && key >= first;
         s_sc[key] = valid ? s : -INFINITY;  // raw dot product; scaled inside the exp2 below
         mx = fmaxf(mx, valid ? s * P.scale_log2e : -INFINITY);
@@ -796,11 +862,13 @@ __global__ void __launch_bounds__(NW * 64) ffa_decode_wg_kernel(const DecodePara
         for (int tile = tile_lo + wave; tile < ntiles; tile += NW) {
             const int key = tile * kWave + lane;
             const float w = s_sc[key];
-            queue_push<T, DH>(acc, sq, w >= 0.f, w, key, vc_bh, vnew, tlen, lane);
+            const int row = beams.v_row(beams.beam(key, tlen), key, tlen, rows_per_sample);
+            queue_push<T, DH>(acc, sq, w >= 0.f, w, row, beams.v_group, vnew, lane);
         }
-        queue_drain<T, DH>(acc, sq, vc_bh, vnew, tlen, lane);
+        queue_drain<T, DH>(acc, sq, beams.v_group, vnew, lane);
     } else {
         for (int tile = tile_lo + wave; tile < ntiles; tile += NW) {
+            const int src = beams.beam(tile * kWave + lane, tlen);  // a row's beam sits in its key's lane
 #pragma unroll 1
             for (int g = 0; g < NVL / VG; ++g) {
                 uint4 vv[VG];
@@ -810,10 +878,13 @@ __global__ void __launch_bounds__(NW * 64) ffa_decode_wg_kernel(const DecodePara
                     // Unconditional loads (rows past the end re-read the new token with
                     // weight 0): a load under a branch would have to be waited for at the
                     // join, one round trip per row.
-                    const int row = tile * kWave + (g * VG + j) * RPI + rg;
+                    const int in_tile = (g * VG + j) * RPI + rg;
+                    const int row = tile * kWave + in_tile;
                     pj[j] = row <= tlen ? s_sc[row] : 0.f;
                     const int r = min(row, tlen);
-                    vv[j] = ld16(r < tlen ? vc_bh + ((size_t)r * NCH + dch) * 16 : vnew + dch * 16);
+                    const char* vb = vc_bh;
+                    if constexpr (BEAM) vb = beams.v_of(__shfl(src, in_tile));
+                    vv[j] = ld16(r < tlen ? vb + ((size_t)r * NCH + dch) * 16 : vnew + dch * 16);
                 }
 #pragma unroll
                 for (int j = 0; j < VG; ++j) fma_chunk(acc, pj[j], vv[j], T{});
@@ -844,7 +915,7 @@ __global__ void __launch_bounds__(NW * 64) ffa_decode_wg_kernel(const DecodePara
 // -- which the pruning rule needs before it may touch a single V row -- then streams only
 // the V rows that survive.  Weights are normalised globally, hence the pieces' partial
 // outputs simply add up (merged by the last piece to arrive).
-template <typename T, int DH, int NW>
+template <typename T, int DH, int NW, bool BEAM>
 __global__ void __launch_bounds__(NW * 64) ffa_scores_kernel(const DecodeParams P) {
     using G = Geo<T, DH>;
     constexpr int NCH = G::NCH;
@@ -883,11 +954,12 @@ __global__ void __launch_bounds__(NW * 64) ffa_scores_kernel(const DecodeParams 
 
     // Each lane keeps a running (max, sum of exp2) over its own keys; lanes, then waves, are
     // folded once at the end.
+    const BeamRows<BEAM> beams(P, b, bh, head_bytes);
     float* sc = P.ws_scores + (size_t)bh * P.score_stride;
     float m_run = -INFINITY, l_run = 0.f;
     for (int tile = tile_lo + wave; tile < tile_hi; tile += NW) {
         const int key = tile * kWave + lane;
-        const float s = tile_qk<T, NCH, G::Q_LDS>(kc_bh, knew, key, tlen, P.Lmax, q_reg, s_q);
+        const float s = tile_qk<T, NCH, G::Q_LDS>(beams.k_of(beams.beam(key, tlen)), knew, key, tlen, P.Lmax, q_reg, s_q);
         const bool valid = key <= tlen && key >= first;
         sc[key] = valid ? s : -INFINITY;  // raw dot product; the whole 64-key tile is written
         if (valid) {
@@ -918,7 +990,7 @@ __global__ void __launch_bounds__(NW * 64) ffa_scores_kernel(const DecodeParams 
     }
 }
 
-template <typename T, int DH, int NW>
+template <typename T, int DH, int NW, bool BEAM>
 __global__ void __launch_bounds__(NW * 64) ffa_pruned_pv_kernel(const DecodeParams P) {
     using G = Geo<T, DH>;
     constexpr int X = G::X, LPR = G::LPR;
@@ -935,9 +1007,10 @@ __global__ void __launch_bounds__(NW * 64) ffa_pruned_pv_kernel(const DecodePara
     step_bounds(P, b, tlen, first);
 
     const size_t head_bytes = (size_t)P.Lmax * DH * sizeof(T);
-    const char* vc_bh = reinterpret_cast<const char*>(P.v_cache) + (size_t)bh * head_bytes;
     const char* vnew = reinterpret_cast<const char*>(P.v) + (size_t)bh * DH * sizeof(T);
     const float* sc = P.ws_scores + (size_t)bh * P.score_stride;
+    const BeamRows<BEAM> beams(P, b, bh, head_bytes);
+    const int rows_per_sample = P.H * P.Lmax;
 
     const int ntiles = tlen / kWave + 1;
     const int tile_first = min(first / kWave, ntiles);  // tiles below are fully masked
@@ -949,8 +1022,9 @@ __global__ void __launch_bounds__(NW * 64) ffa_pruned_pv_kernel(const DecodePara
     // n_splits > 64), all loads in flight at once; every wave of every workgroup of the pair
     // folds them through the same reduction tree, so all arrive at bit-identical M, S ----
     static_assert(kMaxSplits <= 2 * kWave, "two pieces per lane at most");
-    // The first tile's scores travel together with the pieces' (max, sum).
+    // The first tile's scores (and source beams) travel together with the pieces' (max, sum).
     float sr_next = (tile_lo + wave < tile_hi) ? sc[(tile_lo + wave) * kWave + lane] : -INFINITY;
+    int src_next = beams.beam((tile_lo + wave) * kWave + lane, tile_lo + wave < tile_hi ? tlen : 0);
     const float* ml = P.ws_ml + (size_t)bh * P.n_splits * 2;
     float m_a = -INFINITY, l_a = 0.f, m_b = -INFINITY, l_b = 0.f;
     if (lane < P.n_splits) {
@@ -982,7 +1056,9 @@ __global__ void __launch_bounds__(NW * 64) ffa_pruned_pv_kernel(const DecodePara
     for (int tile = tile_lo + wave; tile < tile_hi; tile += NW) {
         const int key = tile * kWave + lane;
         const float sr = sr_next;
+        const int src = src_next;
         sr_next = (tile + NW < tile_hi) ? sc[key + NW * kWave] : -INFINITY;  // one tile ahead
+        src_next = beams.beam(key + NW * kWave, tile + NW < tile_hi ? tlen : 0);
         const float e = (sr == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(fmaf(sr, P.scale_log2e, -M));
         const bool in_range = key >= first && key <= tlen;
         float w;
@@ -999,9 +1075,9 @@ __global__ void __launch_bounds__(NW * 64) ffa_pruned_pv_kernel(const DecodePara
             kept += drop ? 0u : 1u;
             if (P.skip_mask) P.skip_mask[(size_t)bh * P.Lmax + key] = drop ? 1 : 0;
         }
-        queue_push<T, DH>(acc, sq, !drop, w, key, vc_bh, vnew, tlen, lane);
+        queue_push<T, DH>(acc, sq, !drop, w, beams.v_row(src, key, tlen, rows_per_sample), beams.v_group, vnew, lane);
     }
-    queue_drain<T, DH>(acc, sq, vc_bh, vnew, tlen, lane);
+    queue_drain<T, DH>(acc, sq, beams.v_group, vnew, lane);
     if (P.skip_mask && split == 0)  // keys of fully masked leading tiles are dropped too
         for (int i = tid; i < min(tile_first * kWave, tlen); i += NT) P.skip_mask[(size_t)bh * P.Lmax + i] = 1;
 
@@ -1221,11 +1297,11 @@ int static_scratch_address(void** ptr) {
     return FFA_OK;
 }
 
-template <typename T, int DH, int NW>
+template <typename T, int DH, int NW, bool BEAM>
 static int launch_split(const DecodeParams& P, hipStream_t st) {
     const int n_split_heads = P.bh_total - P.n_whole;
     const dim3 grid((unsigned)(P.n_whole + n_split_heads * P.n_splits));
-    hipLaunchKernelGGL((ffa_decode_split_kernel<T, DH, NW>), grid, dim3(NW * 64), 0, st, P);
+    hipLaunchKernelGGL((ffa_decode_split_kernel<T, DH, NW, BEAM>), grid, dim3(NW * 64), 0, st, P);
     if (n_split_heads > 0 && P.n_splits > 1 && P.combine == FFA_COMBINE_KERNEL)
         hipLaunchKernelGGL((ffa_merge_splits_kernel<T, DH>), dim3((unsigned)n_split_heads), dim3(64), 0, st, P);
     return check_launch();
@@ -1248,17 +1324,17 @@ static int launch_split_tpk(const DecodeParams& P, hipStream_t st) {
     }
 }
 
-template <typename T, int DH, int NW>
+template <typename T, int DH, int NW, bool BEAM>
 static int launch_two_pass(const DecodeParams& P, hipStream_t st) {
     const dim3 grid((unsigned)(P.bh_total * P.n_splits));
-    hipLaunchKernelGGL((ffa_scores_kernel<T, DH, NW>), grid, dim3(NW * 64), 0, st, P);
-    hipLaunchKernelGGL((ffa_pruned_pv_kernel<T, DH, NW>), grid, dim3(NW * 64), 0, st, P);
+    hipLaunchKernelGGL((ffa_scores_kernel<T, DH, NW, BEAM>), grid, dim3(NW * 64), 0, st, P);
+    hipLaunchKernelGGL((ffa_pruned_pv_kernel<T, DH, NW, BEAM>), grid, dim3(NW * 64), 0, st, P);
     return check_launch();
 }
 
-template <typename T, int DH, int NW>
+template <typename T, int DH, int NW, bool BEAM>
 static int launch_wg(const DecodeParams& P, size_t lds_bytes, hipStream_t st) {
-    auto kern = ffa_decode_wg_kernel<T, DH, NW>;
+    auto kern = ffa_decode_wg_kernel<T, DH, NW, BEAM>;
     if (lds_bytes > 48 * 1024) {
         // Raise the dynamic-LDS ceiling once per instantiation and device (gfx950: 160 KiB per
         // CU).  The attribute is a property of the loaded function, not of a stream, so the
@@ -1281,10 +1357,10 @@ static int launch_wg(const DecodeParams& P, size_t lds_bytes, hipStream_t st) {
     return check_launch();
 }
 
-template <typename T, int DH>
+template <typename T, int DH, bool BEAM>
 static int dispatch_waves(const DecodeParams& P, const ffa_launch_plan& plan, hipStream_t st) {
     if (plan.kind == FFA_LAUNCH_SPLIT && plan.threads_per_key > 1) {
-        if constexpr (DH == 80) {
+        if constexpr (DH == 80 || BEAM) {  // several lanes per key: own caches only
             return FFA_ERR_PLAN;
         } else {
             const int key = plan.threads_per_key * 100 + plan.waves_per_wg;
@@ -1299,29 +1375,29 @@ static int dispatch_waves(const DecodeParams& P, const ffa_launch_plan& plan, hi
     }
     if (plan.kind == FFA_LAUNCH_SPLIT) {
         switch (plan.waves_per_wg) {
-            case 1: return launch_split<T, DH, 1>(P, st);
-            case 2: return launch_split<T, DH, 2>(P, st);
-            case 4: return launch_split<T, DH, 4>(P, st);
-            case 8: return launch_split<T, DH, 8>(P, st);
+            case 1: return launch_split<T, DH, 1, BEAM>(P, st);
+            case 2: return launch_split<T, DH, 2, BEAM>(P, st);
+            case 4: return launch_split<T, DH, 4, BEAM>(P, st);
+            case 8: return launch_split<T, DH, 8, BEAM>(P, st);
             default: return FFA_ERR_PLAN;
         }
     }
     if (plan.kind == FFA_LAUNCH_TWO_PASS) {
         switch (plan.waves_per_wg) {
-            case 1: return launch_two_pass<T, DH, 1>(P, st);
-            case 2: return launch_two_pass<T, DH, 2>(P, st);
-            case 4: return launch_two_pass<T, DH, 4>(P, st);
-            case 8: return launch_two_pass<T, DH, 8>(P, st);
+            case 1: return launch_two_pass<T, DH, 1, BEAM>(P, st);
+            case 2: return launch_two_pass<T, DH, 2, BEAM>(P, st);
+            case 4: return launch_two_pass<T, DH, 4, BEAM>(P, st);
+            case 8: return launch_two_pass<T, DH, 8, BEAM>(P, st);
             default: return FFA_ERR_PLAN;
         }
     }
     const size_t lds = wg_dynamic_lds_bytes(P.t, plan.waves_per_wg, (int)sizeof(T));
     switch (plan.waves_per_wg) {
-        case 1: return launch_wg<T, DH, 1>(P, lds, st);
-        case 2: return launch_wg<T, DH, 2>(P, lds, st);
-        case 4: return launch_wg<T, DH, 4>(P, lds, st);
-        case 8: return launch_wg<T, DH, 8>(P, lds, st);
-        case 16: return launch_wg<T, DH, 16>(P, lds, st);
+        case 1: return launch_wg<T, DH, 1, BEAM>(P, lds, st);
+        case 2: return launch_wg<T, DH, 2, BEAM>(P, lds, st);
+        case 4: return launch_wg<T, DH, 4, BEAM>(P, lds, st);
+        case 8: return launch_wg<T, DH, 8, BEAM>(P, lds, st);
+        case 16: return launch_wg<T, DH, 16, BEAM>(P, lds, st);
         default: return FFA_ERR_PLAN;
     }
 }
@@ -1329,11 +1405,20 @@ static int dispatch_waves(const DecodeParams& P, const ffa_launch_plan& plan, hi
 template <typename T>
 static int dispatch_head_dim(const DecodeParams& P, int head_dim, const ffa_launch_plan& plan,
                              hipStream_t st) {
+    if (P.cache_indir != nullptr) {
+        switch (head_dim) {
+            case 64: return dispatch_waves<T, 64, true>(P, plan, st);
+            case 80: return dispatch_waves<T, 80, true>(P, plan, st);
+            case 128: return dispatch_waves<T, 128, true>(P, plan, st);
+            case 256: return dispatch_waves<T, 256, true>(P, plan, st);
+            default: return FFA_ERR_HEAD_DIM;
+        }
+    }
     switch (head_dim) {
-        case 64: return dispatch_waves<T, 64>(P, plan, st);
-        case 80: return dispatch_waves<T, 80>(P, plan, st);
-        case 128: return dispatch_waves<T, 128>(P, plan, st);
-        case 256: return dispatch_waves<T, 256>(P, plan, st);
+        case 64: return dispatch_waves<T, 64, false>(P, plan, st);
+        case 80: return dispatch_waves<T, 80, false>(P, plan, st);
+        case 128: return dispatch_waves<T, 128, false>(P, plan, st);
+        case 256: return dispatch_waves<T, 256, false>(P, plan, st);
         default: return FFA_ERR_HEAD_DIM;
     }
 }
@@ -1380,6 +1465,8 @@ int launch_decode(const DecodeArgs& a, const ffa_launch_plan& plan, const Worksp
     P.n_whole = plan.kind == FFA_LAUNCH_SPLIT ? plan.whole_heads : 0;
     P.bh_total = a.B * a.H;
     P.combine = plan.combine;
+    P.cache_indir = a.cache_indir;
+    P.beam_width = a.cache_indir != nullptr ? a.beam_width : 1;
     if (a.precision == FFA_PRECISION_F16) return dispatch_head_dim<uint16_t>(P, a.Dh, plan, st);
     if (a.precision == FFA_PRECISION_BF16) return dispatch_head_dim<bf16_t>(P, a.Dh, plan, st);
     return dispatch_head_dim<float>(P, a.Dh, plan, st);

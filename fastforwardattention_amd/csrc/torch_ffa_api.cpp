@@ -151,7 +151,8 @@ struct FastForwardAttn {
                                torch::Tensor v_cache, float softmax_scale, int curr_timestep,
                                c10::optional<torch::Tensor> seq_lengths, float prob_thresh, int rotary_dim,
                                c10::optional<torch::Tensor> q_bias, c10::optional<torch::Tensor> k_bias,
-                               c10::optional<torch::Tensor> v_bias) {
+                               c10::optional<torch::Tensor> v_bias, c10::optional<torch::Tensor> cache_indir,
+                               int beam_width) {
         const CacheDims d = dims_of(k_cache, v_cache);
         torch::Tensor bias[3];
         const c10::optional<torch::Tensor>* in[3] = {&q_bias, &k_bias, &v_bias};
@@ -162,10 +163,20 @@ struct FastForwardAttn {
             bias[i] = token_input(in[i]->value(), k_cache, (int64_t)d.H * d.Dh, "bias");
             *slot[i] = bias[i].data_ptr();
         }
-        torch::Tensor sl;
+        torch::Tensor sl, indir;
         if (seq_lengths.has_value()) sl = seq_lengths.value();
+        ffa_beam_indirection beams = {nullptr, beam_width};
+        if (cache_indir.has_value()) {
+            indir = cache_indir.value();
+            TORCH_CHECK(indir.device() == k_cache.device() && indir.scalar_type() == torch::kInt &&
+                            indir.is_contiguous() && indir.dim() == 2 && indir.size(0) == d.B &&
+                            indir.size(1) == d.Lmax,
+                        "ff_attention: cache_indir must be a contiguous int32 tensor [B, max_len] on the cache's device");
+            beams.cache_indir = indir.data_ptr<int>();
+        }
         return run(q, k, v, k_cache, v_cache, softmax_scale, curr_timestep, seq_lengths.has_value() ? &sl : nullptr,
-                   prob_thresh, !seq_lengths.has_value(), nullptr, nullptr, &tt);
+                   prob_thresh, !seq_lengths.has_value(), nullptr, nullptr, &tt,
+                   cache_indir.has_value() ? &beams : nullptr);
     }
 
     // Not in the reference: the same step plus what pruning dropped.
@@ -210,7 +221,8 @@ private:
     torch::Tensor run(const torch::Tensor& q_in, const torch::Tensor& k_in, const torch::Tensor& v_in,
                       torch::Tensor& kc, torch::Tensor& vc, float softmax_scale, int t,
                       const torch::Tensor* seq_lengths, float prob_thresh, bool right_or_no_padding,
-                      torch::Tensor* kept, torch::Tensor* mask, const ffa_token_transform* transform = nullptr) {
+                      torch::Tensor* kept, torch::Tensor* mask, const ffa_token_transform* transform = nullptr,
+                      const ffa_beam_indirection* beams = nullptr) {
         TORCH_CHECK(kc.is_cuda() && vc.is_cuda() && kc.device() == vc.device() &&
                         kc.scalar_type() == vc.scalar_type(),
                     "ff_attention: caches must be GPU tensors of one dtype on one device");
@@ -240,14 +252,17 @@ private:
         ffa_launch_plan plan;
         const bool diag = kept != nullptr || mask != nullptr;
         // The default launch keeps diagnostics at any length; the exact split kernel has none.
-        check_status(ffa_plan_launch(plan_precision(precision), d.B, d.H, d.Dh, t, prob_thresh,
-                                     (ft_kernel_launch || diag) ? 1 : 0, 0, &plan),
+        // Plans with several lanes per key (only the measured table holds such) take no beam
+        // indirection: with one, plan by the rules alone.
+        check_status((beams != nullptr ? ffa_plan_launch_rules : ffa_plan_launch)(
+                         plan_precision(precision), d.B, d.H, d.Dh, t, prob_thresh,
+                         (ft_kernel_launch || diag) ? 1 : 0, 0, &plan),
                      "launch planning");
-        if (transform != nullptr) {
-            TORCH_CHECK(!diag, "ff_attention: diagnostics and a token transform cannot be combined");
+        if (transform != nullptr || beams != nullptr) {
+            TORCH_CHECK(!diag, "ff_attention: diagnostics cannot be combined with a token transform or beams");
             check_status(ffa_attention_ex(precision, d.B, d.H, d.Dh, d.Lmax, softmax_scale, t, q.data_ptr(),
                                           k.data_ptr(), v.data_ptr(), kc.data_ptr(), vc.data_ptr(), out.data_ptr(),
-                                          sl_ptr, prob_thresh, &plan, right_or_no_padding ? 1 : 0, transform,
+                                          sl_ptr, prob_thresh, &plan, right_or_no_padding ? 1 : 0, transform, beams,
                                           workspace.data_ptr(), (size_t)workspace.numel(), stream_of(kc)),
                          "attention");
             return out;
@@ -281,7 +296,12 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
                                float, int, torch::Tensor, float>(&FastForwardAttn::attention),
              "Attention forward, left-padded batch")
         .def("attention_ex", &FastForwardAttn::attention_ex,
-             "Attention forward with q/k/v bias and rotary embedding of the new token")
+             "Attention forward with q/k/v bias and rotary embedding of the new token and, optionally, "
+             "beam-search cache indirection (cache_indir int32 [B, max_len], beam_width)",
+             py::arg("q"), py::arg("k"), py::arg("v"), py::arg("k_cache"), py::arg("v_cache"),
+             py::arg("softmax_scale"), py::arg("curr_timestep"), py::arg("seq_lengths"), py::arg("prob_thresh"),
+             py::arg("rotary_dim"), py::arg("q_bias"), py::arg("k_bias"), py::arg("v_bias"),
+             py::arg("cache_indir") = py::none(), py::arg("beam_width") = 1)
         .def("attention_diag", &FastForwardAttn::attention_diag,
              "Attention forward plus (kept_count, skip_mask) of the pruning rule")
         .def("launch_plan", &FastForwardAttn::launch_plan, "Launch plan for (t, p)");

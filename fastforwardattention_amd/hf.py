@@ -20,6 +20,13 @@ Written against the installed transformers (5.x) instead of a patched copy of it
   (`attention_ex(..., rotary_dim, ...)`: the FasterTransformer feature of attention.cu:874-882):
   the layer's forward is wrapped and skips the torch-side sin/cos gather, split, rotate and
   concatenate.  `enable(model, fused_rotary=False)` keeps the reference's arrangement.
+* beam search (`generate(num_beams=n, past_key_values=FFACache(..., num_beams=n))`): where the
+  reference's models copy every layer's caches along the batch axis after each step
+  (`_reorder_cache`, modeling_opt.py:1072-1075, modeling_gptj.py:911-918), the cache keeps one
+  small table per layer -- for every sample and slot, the beam of the group whose caches hold
+  that slot -- permutes its rows when beams are re-parented, and hands it to the engine
+  (`attention_ex(..., cache_indir, beam_width)`: the FasterTransformer feature of
+  attention.cu:1024-1033 that the reference switches off).  Keys and values never move.
 
     from fastforwardattention_amd import hf
     hf.enable(model)
@@ -56,10 +63,14 @@ class FFALayer(CacheLayerMixin):
     is_compileable = False
 
     def __init__(self, max_new_tokens: int, prob_thresh: float = 0.0,
-                 use_default_kernel_launch: bool = False, engine=None):
+                 use_default_kernel_launch: bool = False, engine=None, num_beams: int = 1):
         super().__init__()
         if max_new_tokens < 1:
             raise ValueError("max_new_tokens must be >= 1")
+        if num_beams < 1:
+            raise ValueError("num_beams must be >= 1")
+        self.num_beams = int(num_beams)
+        self.beam_table = None      # int32 [B, max_len]: beam of the group whose caches hold the slot
         self.max_new_tokens = int(max_new_tokens)
         self.prob_thresh = float(prob_thresh)
         self.use_default_kernel_launch = bool(use_default_kernel_launch)
@@ -100,14 +111,32 @@ class FFALayer(CacheLayerMixin):
         return -1
 
     def reset(self):
-        self.engine, self.t, self.max_len, self.first_key = None, 0, 0, None
+        self.engine, self.t, self.max_len, self.first_key, self.beam_table = None, 0, 0, None, None
         self._hooked = self._pending = False
 
-    def _unsupported(self, *a, **k):
-        raise NotImplementedError("FFACache holds the reference's fixed-layout caches: no beam reordering, "
-                                  "cropping or batch reshaping (the reference disables cache_indir too)")
+    def reorder_cache(self, beam_idx):
+        """Beam search re-parents the samples: sample b continues sample beam_idx[b] of its own
+        group.  Its history becomes the parent's -- a row copy in the table -- and the slot
+        the parent wrote last (t - 1) is found in the parent's own caches."""
+        if self.engine is None:
+            return
+        if self.num_beams == 1:
+            raise NotImplementedError("FFACache: beam search needs FFACache(..., num_beams=n) with generate's "
+                                      "num_beams (the caches are not copied between samples)")
+        beam_idx = beam_idx.to(self.beam_table.device)
+        B = self.beam_table.shape[0]
+        own = torch.arange(B, device=beam_idx.device)
+        if beam_idx.numel() != B or bool(((beam_idx // self.num_beams) != (own // self.num_beams)).any()):
+            raise ValueError("FFACache: a beam can only continue a beam of its own group")
+        table = self.beam_table.index_select(0, beam_idx)
+        table[:, self.t - 1] = (beam_idx % self.num_beams).to(torch.int32)
+        self.beam_table = table
 
-    reorder_cache = crop = batch_repeat_interleave = batch_select_indices = offload = prefetch = _unsupported
+    def _unsupported(self, *a, **k):
+        raise NotImplementedError("FFACache holds the reference's fixed-layout caches: no cropping or batch "
+                                  "reshaping")
+
+    crop = batch_repeat_interleave = batch_select_indices = offload = prefetch = _unsupported
 
     # -- the two passes -------------------------------------------------------------------
     def _prompt_pass(self, key_states, value_states):
@@ -122,6 +151,14 @@ class FFALayer(CacheLayerMixin):
         self.engine = cls(key_states.contiguous(), value_states.to(key_states.dtype).contiguous(),
                           self.max_len, self.use_default_kernel_launch)
         self.t = prompt_len
+        if self.num_beams > 1:
+            B = key_states.shape[0]
+            if B % self.num_beams:
+                raise ValueError(f"FFACache: batch {B} is not a multiple of num_beams = {self.num_beams}")
+            if not hasattr(self.engine, "attention_ex"):
+                raise NotImplementedError("FFACache: this engine has no attention_ex, which beam search needs")
+            own = (torch.arange(B, device=key_states.device) % self.num_beams).to(torch.int32)
+            self.beam_table = own[:, None].expand(B, self.max_len).contiguous()   # every slot in the sample's own caches
         setattr(key_states, _TAG, self)
         return key_states, value_states
 
@@ -144,7 +181,11 @@ class FFALayer(CacheLayerMixin):
         dt = self.dtype
         q, k, v = query.to(dt), key.to(dt), value.to(dt)
         k_cache, v_cache = self.engine.get_cache()
-        if self.first_key is None:
+        if self.beam_table is not None:
+            out = self.engine.attention_ex(q, k, v, k_cache, v_cache, float(scale), self.t, self.first_key,
+                                           self.prob_thresh, 0, None, None, None,
+                                           cache_indir=self.beam_table, beam_width=self.num_beams)
+        elif self.first_key is None:
             out = self.engine.attention(q, k, v, k_cache, v_cache, float(scale), self.t, self.prob_thresh)
         else:
             out = self.engine.attention(q, k, v, k_cache, v_cache, float(scale), self.t, self.first_key,
@@ -163,8 +204,9 @@ class FFALayer(CacheLayerMixin):
             raise RuntimeError(f"FFACache: cache full ({self.max_len} slots = prompt + max_new_tokens)")
         dt = self.dtype
         k_cache, v_cache = self.engine.get_cache()
+        beams = {} if self.beam_table is None else dict(cache_indir=self.beam_table, beam_width=self.num_beams)
         out = self.engine.attention_ex(query.to(dt), key.to(dt), value.to(dt), k_cache, v_cache, float(scale), self.t,
-                                       self.first_key, self.prob_thresh, int(rotary_dim), None, None, None)
+                                       self.first_key, self.prob_thresh, int(rotary_dim), None, None, None, **beams)
         self.t += 1
         return out
 
@@ -173,12 +215,13 @@ class FFACache(Cache):
     """`past_key_values` object that keeps every layer's keys and values inside a
     `FastForwardAttn` (cache layouts [B,H,Dh/x,Lmax,x] / [B,H,Lmax,Dh], Lmax = prompt +
     max_new_tokens).  `engine` replaces the `FastForwardAttn` class (same constructor and
-    methods); tests use it to run the bookkeeping without a GPU."""
+    methods); tests use it to run the bookkeeping without a GPU.  num_beams: generate's num_beams
+    when beam search is used (samples are grouped num_beams at a time, as generate lays them out)."""
 
     def __init__(self, max_new_tokens: int, prob_thresh: float = 0.0,
-                 use_default_kernel_launch: bool = False, engine=None):
+                 use_default_kernel_launch: bool = False, engine=None, num_beams: int = 1):
         super().__init__(layer_class_to_replicate=functools.partial(
-            FFALayer, max_new_tokens, prob_thresh, use_default_kernel_launch, engine))
+            FFALayer, max_new_tokens, prob_thresh, use_default_kernel_launch, engine, num_beams))
 
     @classmethod
     def from_env(cls, engine=None):

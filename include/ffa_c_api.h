@@ -48,8 +48,10 @@ typedef enum ffa_status {
     FFA_ERR_NO_DEVICE = 12,     /* no usable gfx950 device / HIP runtime error               */
     FFA_ERR_SCRATCH_LIMIT = 13, /* ffa_attention_static_scratch: the plan needs more scratch */
                                 /* than FFA_STATIC_SCRATCH_BYTES                             */
-    FFA_ERR_TRANSFORM = 14      /* rotary_embedding_dim odd, negative or > head_dim, or a    */
+    FFA_ERR_TRANSFORM = 14,     /* rotary_embedding_dim odd, negative or > head_dim, or a    */
                                 /* bias pointer not 16-byte aligned                          */
+    FFA_ERR_BEAM = 15           /* beam indirection: NULL or misaligned table, beam_width    */
+                                /* < 1 or not a divisor of batch_size, or a group too large   */
 } ffa_status;
 
 /* precision codes: the same integers the reference passes to get_launch_params
@@ -192,7 +194,8 @@ int ffa_attention_diag(int precision, int batch_size, int head_num, int head_dim
  * The decode step with the FasterTransformer features that the reference's kernel carries but
  * its host code switches off (attention.cu:1472-1483): q/k/v bias (attention.cu:856-873,
  * :1157-1158, :1242), rotary position embedding of q and k (attention.cu:874-882;
- * decoder_masked_multihead_attention_utils.h:1137-1160) and a bf16 element type.
+ * decoder_masked_multihead_attention_utils.h:1137-1160), the beam-search cache indirection
+ * and a bf16 element type.
  *   precision  FFA_PRECISION_F16 | FFA_PRECISION_F32 | FFA_PRECISION_BF16 (bf16 caches are built
  *              with ffa_init_cache_f16: cache construction only moves 16-byte chunks);
  *   transform  NULL = none (then the call equals ffa_attention_f16 / _f32).  Otherwise, before
@@ -206,6 +209,20 @@ int ffa_attention_diag(int precision, int batch_size, int head_num, int head_dim
  *              supports no padded batch, attention.cu:879).  The transformed k and v are what
  *              the caches receive.  It runs as one small kernel ahead of the decode kernel on
  *              the same stream; its output lives in the workspace.
+ *   beams      NULL = none.  Otherwise beam-search cache indirection (attention.cu:779-793,
+ *              :1003, :1024-1033, :1143, :1195-1202; the reference's host code passes nullptr
+ *              and beam_width 1, attention.cu:1477-1479): sample b is beam b % beam_width of
+ *              group b / beam_width, and its cached key i < t is read from the caches of
+ *              sample (b - b % beam_width) + cache_indir[b * max_seq_len + i] instead of its own;
+ *              the new token is appended to the sample's own caches as always.  A search then
+ *              re-parents beams by permuting rows of this small table instead of copying
+ *              caches.  Entries outside [0, beam_width) are clamped into that range.  All
+ *              beams of a group must be at the same length (same t, same seq_lengths entry):
+ *              a beam's slot t is written in the launch in which its siblings read the slots
+ *              below theirs.  batch_size must be a multiple of beam_width and
+ *              beam_width * head_num * max_seq_len must stay below 2^31 (FFA_ERR_BEAM);
+ *              launch plans with more than one lane per key do not take an indirection
+ *              (FFA_ERR_PLAN; a NULL plan never picks one).
  */
 typedef struct ffa_token_transform {
     const void* q_bias;
@@ -215,12 +232,17 @@ typedef struct ffa_token_transform {
     float rotary_base;            /* 10000 in the reference (utils.h:1139); <= 0 selects that  */
 } ffa_token_transform;
 
+typedef struct ffa_beam_indirection {
+    const int32_t* cache_indir; /* device, [batch_size, max_seq_len]: source beam of each key */
+    int32_t beam_width;         /* samples per group, >= 1                                    */
+} ffa_beam_indirection;
+
 int ffa_attention_ex(int precision, int batch_size, int head_num, int head_dim, int max_seq_len,
                      float softmax_scale, int t, const void* q, const void* k, const void* v,
                      void* k_cache, void* v_cache, void* out, const int* seq_lengths,
                      float prob_thresh, const ffa_launch_plan* plan, int right_or_no_padding,
-                     const ffa_token_transform* transform, void* workspace, size_t workspace_bytes,
-                     void* stream);
+                     const ffa_token_transform* transform, const ffa_beam_indirection* beams,
+                     void* workspace, size_t workspace_bytes, void* stream);
 
 /*
  * The same step for callers that cannot allocate device memory (code under HIP graph

@@ -12,6 +12,7 @@ citations are file:line under the reference checkout.
   pack_v_cache          attention.cu:1593-1608            [B,H,L,Dh] -> [B,H,Lmax,Dh]
   append_kv             attention.cu:901-914, :1246       write slot t of both caches
   decode_step           attention.cu:805-817, :1054, :1072, :1111-1116 (masking)
+  beam_keys_values      attention.cu:779-793, :1003, :1024-1033, :1143, :1195-1202 (cache_indir)
   half_from_ushort_rn   cuda_fp16.h __half(unsigned short) == __ushort2half_rn
   leq_f16_bits          attention.cu:466-469              __hle on converted bit patterns
   pruned_decode_step    attention.cu:1108-1126, :1184-1191, :1227-1256
@@ -29,6 +30,12 @@ Pinning status (what independent evidence fixes each function):
                      pinned: known answers of IEEE round-to-nearest-even at 11 significant
                      bits (2049->2048, 2051->2052, 65520->inf) and exhaustive comparison
                      with numpy's own uint16->float16 cast over all 65536 patterns.
+  beam_keys_values   pinned: the identity table reproduces the plain step bit for bit; a
+                     simulated beam search that re-parents beams by permuting table rows
+                     gives, step by step, bit-identical outputs to one that copies whole
+                     caches the way the reference's models do (_reorder_cache,
+                     modeling_opt.py:1072-1075); an element-by-element Python loop over the
+                     reference's flat offsets on a tiny case.
   token_transform    pinned: the installed transformers' GPT-J apply_rotary_pos_emb /
                      create_sinusoidal_positions on fp32 tensors (same pairs, signs and
                      angles), a rotation's invariants (norm of every pair, position 0 is
@@ -122,10 +129,37 @@ def _bounds(B, t, seq_lengths, right_or_no_padding):
     return np.full(B, t, np.int64), sl.copy()
 
 
+def beam_keys_values(k_cache, v_cache, b, n, cache_indir=None, beam_width=1):
+    """Keys and values 0..n-1 that sample b attends over, as (K [H,n,Dh], V [H,n,Dh]); slot
+    n-1 holds the token just appended.
+
+    Without a table: the sample's own caches.  With one (beam search): sample b is beam
+    b % beam_width of group bbi = b // beam_width (attention.cu:785-787); key ti < n-1 is read
+    from sample bbi*beam_width + cache_indir[b*Lmax + ti] (attention.cu:1003, :1024-1033 for K,
+    :1143, :1195-1202 for V -- the base pointer is the group's first beam, the table entry an
+    offset of whole samples from it); the new token (ti = n-1) never goes through the table:
+    it is taken from the registers that also write it to the sample's own slot
+    (attention.cu:901-914, :1227-1256)."""
+    B, H, C, Lmax, x = k_cache.shape
+    if cache_indir is None:
+        return unpack_k_cache(k_cache[b:b + 1], n)[0], v_cache[b, :, :n, :]
+    indir = np.asarray(cache_indir).reshape(B, Lmax)
+    bbi = b // beam_width
+    src = np.full(n, b, np.int64)
+    src[:n - 1] = bbi * beam_width + indir[b, :n - 1]
+    K = np.empty((H, n, C * x), k_cache.dtype)
+    V = np.empty((H, n, C * x), v_cache.dtype)
+    for ti in range(n):
+        K[:, ti, :] = k_cache[src[ti], :, :, ti, :].reshape(H, C * x)
+        V[:, ti, :] = v_cache[src[ti], :, ti, :]
+    return K, V
+
+
 def decode_step(q, k, v, k_cache, v_cache, scale, t, seq_lengths=None,
-                right_or_no_padding=True, acc=np.float32):
+                right_or_no_padding=True, acc=np.float32, cache_indir=None, beam_width=1):
     """One exact (p = 0) decode step: append k,v at slot tlength[b], attend over keys
-    first_key[b] .. tlength[b].  Mutates the caches.  Returns out [B,H,Dh] in `acc`."""
+    first_key[b] .. tlength[b] (read through `cache_indir` when given, see beam_keys_values).
+    Mutates the caches.  Returns out [B,H,Dh] in `acc`."""
     B, H, C, Lmax, x = k_cache.shape
     Dh = C * x
     tlen, first = _bounds(B, t, seq_lengths, right_or_no_padding)
@@ -134,8 +168,7 @@ def decode_step(q, k, v, k_cache, v_cache, scale, t, seq_lengths=None,
     out = np.zeros((B, H, Dh), dtype=acc)
     for b in range(B):
         n = int(tlen[b]) + 1
-        Kb = unpack_k_cache(k_cache[b:b + 1], n)[0]
-        Vb = v_cache[b, :, :n, :]
+        Kb, Vb = beam_keys_values(k_cache, v_cache, b, n, cache_indir, beam_width)
         if first[b] > tlen[b]:
             continue  # every key masked: sum = 0, all logits 0 -> out = 0 (attention.cu:1113)
         out[b] = attn_closed_form(q[b], Kb, Vb, scale,
@@ -244,7 +277,7 @@ def rotary_positions(B, t, seq_lengths=None, right_or_no_padding=True) -> np.nda
 
 # --------------------------------------------------------------------------- pruning rule
 def pruned_decode_step(q, k, v, k_cache, v_cache, scale, t, p, seq_lengths=None,
-                       right_or_no_padding=True, elem=None):
+                       right_or_no_padding=True, elem=None, cache_indir=None, beam_width=1):
     """One decode step with threshold-p pruning, transcribed from attention.cu.
 
     Per (b,h), with e_i = exp(s_i - max over unmasked s) (0 if masked, :1111-1116),
@@ -257,6 +290,8 @@ def pruned_decode_step(q, k, v, k_cache, v_cache, scale, t, p, seq_lengths=None,
     Scores s_i, the P.V products and their sum are carried in fp32 here (the reference
     carries them in T; this build's contract is fp32 accumulation), the result is
     returned in fp32 before the final rounding to T.
+
+    Keys are read through `cache_indir` when given (beam_keys_values).
 
     elem = "bf16" (caches passed as fp32 arrays of bf16 values): T-rounding to bf16 and a
     numeric P_i <= thr; the reference has no bf16 behaviour to follow (ENABLE_BF16 is never
@@ -277,8 +312,8 @@ def pruned_decode_step(q, k, v, k_cache, v_cache, scale, t, p, seq_lengths=None,
     thr_all = np.zeros((B, H), f32)
     for b in range(B):
         n = int(tlen[b]) + 1
-        Kb = unpack_k_cache(k_cache[b:b + 1], n)[0].astype(f32)        # [H,n,Dh]
-        Vb = v_cache[b, :, :n, :].astype(f32)
+        Kb, Vb = beam_keys_values(k_cache, v_cache, b, n, cache_indir, beam_width)   # [H,n,Dh]
+        Kb, Vb = Kb.astype(f32), Vb.astype(f32)
         s = (np.einsum("hd,hnd->hn", q[b], Kb).astype(f32) * f32(scale)).astype(f32)
         masked = np.arange(n)[None, :] < first[b]
         masked = np.broadcast_to(masked, s.shape)

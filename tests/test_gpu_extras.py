@@ -1,5 +1,5 @@
-"""GPU parity of ffa_attention_ex: the bf16 element type and the new-token transform (q/k/v bias,
-rotary embedding), through the C ABI, against the CPU oracle.
+"""GPU parity of ffa_attention_ex: the bf16 element type, the new-token transform (q/k/v bias,
+rotary embedding) and the beam-search cache indirection, through the C ABI, against the CPU oracle.
 
 Tolerances.  fp16 / fp32 outputs: 1e-3 / 1e-6 max-abs against the float64 closed form, as in the
 other parity tests.  bf16 outputs: one bf16 ulp of the closed form (|err| <= 2^-7 |want| + 1e-5;
@@ -62,7 +62,7 @@ class ExSession:
         torch.cuda.synchronize()
 
     def step(self, q, k, v, scale, t, p=0.0, plan=None, seq_lengths=None, rnp=True, transform=None,
-             expect=capi.FFA_OK):
+             beams=None, expect=capi.FFA_OK):
         qd, kd, vd = (_to_dev(a, self.elem) for a in (q, k, v))
         out = torch.full((self.B, self.H, self.Dh), float("nan"), dtype=ELEMS[self.elem][1], device="cuda:0")
         sl = None if seq_lengths is None else torch.from_numpy(np.asarray(seq_lengths, np.int32)).to("cuda:0")
@@ -76,10 +76,17 @@ class ExSession:
                     setattr(tt, name, keep[-1].data_ptr())
             tt.rotary_embedding_dim = transform.get("rotary_dim", 0)
             tt.rotary_base = transform.get("base", 0.0)
+        bi = None
+        if beams is not None:                      # (table [B, Lmax] or None, beam_width)
+            table, bw = beams
+            if table is not None:
+                keep.append(torch.from_numpy(np.ascontiguousarray(table, np.int32)).to("cuda:0"))
+            bi = capi.BeamIndirection(keep[-1].data_ptr() if table is not None else None, bw)
         rc = self.lib.ffa_attention_ex(self.precision, self.B, self.H, self.Dh, self.Lmax, float(scale), int(t),
                                        ptr(qd), ptr(kd), ptr(vd), ptr(self.k_cache), ptr(self.v_cache), ptr(out),
                                        ptr(sl), float(p), C.byref(plan) if plan is not None else None, int(rnp),
-                                       C.byref(tt) if tt is not None else None, ptr(self.ws), self.ws.numel(), None)
+                                       C.byref(tt) if tt is not None else None,
+                                       C.byref(bi) if bi is not None else None, ptr(self.ws), self.ws.numel(), None)
         assert rc == expect, capi.STATUS_NAMES.get(rc, rc)
         torch.cuda.synchronize()
         return None if rc != capi.FFA_OK else out.float().cpu().numpy()
@@ -284,8 +291,156 @@ def test_transform_argument_validation():
     x = _to_dev(q, "f16")
     tt = capi.TokenTransform(rotary_embedding_dim=32)
     rc = sess.lib.ffa_attention_ex(16, B, H, Dh, L + 1, 0.125, L, ptr(x), ptr(x), ptr(x), ptr(sess.k_cache),
-                                   ptr(sess.v_cache), ptr(x), None, 0.0, None, 1, C.byref(tt), ptr(tiny), 64, None)
+                                   ptr(sess.v_cache), ptr(x), None, 0.0, None, 1, C.byref(tt), None, ptr(tiny), 64, None)
     assert rc == capi.FFA_ERR_WORKSPACE          # no room for the transformed token
     rc = sess.lib.ffa_attention_ex(12, B, H, Dh, L + 1, 0.125, L, ptr(x), ptr(x), ptr(x), ptr(sess.k_cache),
-                                   ptr(sess.v_cache), ptr(x), None, 0.0, None, 1, None, ptr(sess.ws), sess.ws.numel(), None)
+                                   ptr(sess.v_cache), ptr(x), None, 0.0, None, 1, None, None, ptr(sess.ws), sess.ws.numel(),
+                                   None)
     assert rc == capi.FFA_ERR_DTYPE
+
+
+# ------------------------------------------------------------------ beam-search cache indirection
+def _cache_values(sess):
+    """The session's caches as fp32 value arrays (k in chunk layout, v)."""
+    return sess.k_cache.float().cpu().numpy(), sess.v_cache.float().cpu().numpy()
+
+
+@pytest.mark.parametrize("elem,Dh", [("f16", 64), ("f16", 80), ("f16", 256), ("f32", 64), ("f32", 128), ("bf16", 128)])
+@pytest.mark.parametrize("t", [0, 63, 500])
+def test_beam_indirection_exact_step_all_plans(elem, Dh, t):
+    """A random table (every key of every beam from a random sibling), every plan kind.  The
+    output follows the table; the new token lands in the sample's own caches, nothing else
+    in the caches changes."""
+    groups, bw, H = 2, 3, 2
+    B, Lmax = groups * bw, t + 3
+    rng, K, V, q, k, v = _inputs(9000 + Dh + t, B, H, t, Dh, elem)
+    scale = 1.0 / np.sqrt(Dh)
+    table = rng.integers(0, bw, (B, Lmax)).astype(np.int32)
+    kc0, vc0 = _pack(K, V, Lmax, elem)
+    want = O.decode_step(q, k, v, kc0, vc0, scale, t, acc=np.float64, cache_indir=table, beam_width=bw)
+    if t > 0:
+        plain = O.decode_step(q, k, v, *_pack(K, V, Lmax, elem), scale, t, acc=np.float64)
+        assert np.abs(want - plain).max() > 1e-2          # the table matters
+    prec = 16 if elem != "f32" else 32
+    for name, plan in _plans(prec, B, H, Dh, t) + [("library", None)]:
+        _say("beams", elem, Dh, t, name)
+        sess = ExSession(K, V, Lmax, elem)
+        if plan is not None and plan.threads_per_key > 1:
+            sess.step(q, k, v, scale, t, plan=plan, beams=(table, bw), expect=capi.FFA_ERR_PLAN)
+            continue
+        got = sess.step(q, k, v, scale, t, plan=plan, beams=(table, bw))
+        assert (np.abs(got - want) <= _out_tol(want, elem)).all(), (name, float(np.abs(got - want).max()))
+        kc, vc = _cache_values(sess)
+        np.testing.assert_array_equal(kc, kc0, err_msg=name)
+        np.testing.assert_array_equal(vc, vc0, err_msg=name)
+
+
+@pytest.mark.parametrize("padding", ["left", "right"])
+def test_beam_indirection_with_padding(padding):
+    groups, bw, H, Dh, L, elem = 3, 2, 4, 64, 300, "f16"
+    B, Lmax = groups * bw, L + 2
+    rng, K, V, q, k, v = _inputs(9100, B, H, L, Dh, elem)
+    table = rng.integers(0, bw, (B, Lmax)).astype(np.int32)
+    if padding == "left":
+        sl, rnp = rng.integers(0, L // 2, B), False
+    else:
+        sl, rnp = np.repeat(rng.integers(L // 2, L + 1, groups), bw), True   # one length per group
+    kc0, vc0 = _pack(K, V, Lmax, elem)
+    want = O.decode_step(q, k, v, kc0, vc0, 0.125, L, seq_lengths=sl, right_or_no_padding=rnp, acc=np.float64,
+                         cache_indir=table, beam_width=bw)
+    for name, plan in _plans(16, B, H, Dh, L) + [("library", None)]:
+        if plan is not None and plan.threads_per_key > 1:
+            continue
+        _say("beams padding", padding, name)
+        sess = ExSession(K, V, Lmax, elem)
+        got = sess.step(q, k, v, 0.125, L, plan=plan, seq_lengths=sl, rnp=rnp, beams=(table, bw))
+        assert np.abs(got - want).max() <= 1e-3, name
+        kc, vc = _cache_values(sess)
+        np.testing.assert_array_equal(kc, kc0, err_msg=name)
+        np.testing.assert_array_equal(vc, vc0, err_msg=name)
+
+
+@pytest.mark.parametrize("elem", ["f16", "f32"])
+def test_beam_indirection_pruned_step(elem):
+    """p > 0 through the table: one-workgroup and two-pass kernels.  The skip set is not returned
+    by ffa_attention_ex, so keys whose probability sits within a rounding of the threshold may
+    fall either way: their weight is the slack of the comparison."""
+    groups, bw, H, Dh, L, p = 2, 2, 3, 64, 900, 1e-2
+    B, Lmax = groups * bw, L + 1
+    rng, K, V, q, k, v = _inputs(9200, B, H, L, Dh, elem)
+    qd = q / np.linalg.norm(q, axis=-1, keepdims=True)
+    table = rng.integers(0, bw, (B, Lmax)).astype(np.int32)
+    for b in range(B):                                   # peaked keys, placed where sample b reads them
+        for h in range(H):
+            for pos in rng.choice(L, 16, replace=False):
+                src = (b // bw) * bw + table[b, pos]
+                K[src, h, pos] = O.round_to(4 * qd[b, h] + 0.1 * rng.standard_normal(Dh), elem)
+    kc0, vc0 = _pack(K, V, Lmax, elem)
+    dt = np.float16 if elem == "f16" else np.float32
+    want, skip, P, thr = O.pruned_decode_step(q, k, v, kc0.astype(dt), vc0.astype(dt), 0.125, L, p,
+                                              cache_indir=table, beam_width=bw)
+    assert 0.1 < skip[:, :, :L].mean() < 0.999
+    near = np.abs(P - thr[:, :, None]) <= 2.0 ** -9 * thr[:, :, None]
+    Vread = np.stack([O.beam_keys_values(kc0, vc0, b, L, table, bw)[1] for b in range(B)])   # [B,H,L,Dh]
+    slack = np.einsum("bhn,bhnd->bhd", np.where(near[:, :, :L], P[:, :, :L], 0), np.abs(Vread))
+    ntiles = L // 64 + 1
+    for plan in (capi.make_plan(capi.FFA_LAUNCH_WORKGROUP, 2, 1, ntiles), capi.make_plan(capi.FFA_LAUNCH_WORKGROUP, 16, 1, ntiles),
+                 capi.make_plan(capi.FFA_LAUNCH_TWO_PASS, 4, -(-ntiles // 3), 3), None):
+        _say("beams pruned", elem, plan)
+        sess = ExSession(K, V, Lmax, elem)
+        got = sess.step(q, k, v, 0.125, L, p=p, plan=plan, beams=(table, bw))
+        assert (np.abs(got - want) <= (1e-3 if elem == "f16" else 1e-5) + slack).all(), plan
+
+
+def test_beam_search_by_table_on_the_gpu_equals_search_by_cache_copy():
+    """The toy beam search of the oracle's own pinning test, table side on the GPU: caches are
+    never copied, rows of the table are; against the oracle searching by cache copy."""
+    groups, bw, H, Dh, L, steps, elem = 2, 4, 8, 64, 130, 70, "f16"
+    B, Lmax = groups * bw, L + steps
+    rng, K, V, *_ = _inputs(9300, B, H, L, Dh, elem)
+    sess = ExSession(K, V, Lmax, elem)
+    kc, vc = _pack(K, V, Lmax, elem)
+    table = np.repeat((np.arange(B) % bw)[:, None], Lmax, 1).astype(np.int32)
+    for s in range(steps):
+        t = L + s
+        q, k, v = (O.round_to(rng.standard_normal((B, H, Dh)), elem) for _ in range(3))
+        got = sess.step(q, k, v, 0.125, t, beams=(table, bw))
+        want = O.decode_step(q, k, v, kc, vc, 0.125, t, acc=np.float64)
+        assert np.abs(got - want).max() <= 1e-3, s
+        parent = (np.arange(B) // bw) * bw + rng.integers(0, bw, B)
+        kc, vc = kc[parent].copy(), vc[parent].copy()
+        table = table[parent].copy()
+        table[:, t] = parent % bw
+
+
+def test_beam_argument_validation():
+    B, H, Dh, L = 4, 2, 64, 20
+    rng, K, V, q, k, v = _inputs(9400, B, H, L, Dh, "f16")
+    sess = ExSession(K, V, L + 1, "f16")
+    table = np.zeros((B, L + 1), np.int32)
+    sess.step(q, k, v, 0.125, L, beams=(None, 2), expect=capi.FFA_ERR_BEAM)      # no table
+    sess.step(q, k, v, 0.125, L, beams=(table, 0), expect=capi.FFA_ERR_BEAM)
+    sess.step(q, k, v, 0.125, L, beams=(table, 3), expect=capi.FFA_ERR_BEAM)     # 4 % 3 != 0
+    # entries outside [0, beam_width) are clamped, never followed out of the group
+    wild = np.where(rng.random((B, L + 1)) < 0.5, -7, 1000).astype(np.int32)
+    got = sess.step(q, k, v, 0.125, L, beams=(wild, 2))
+    kc0, vc0 = _pack(K, V, L + 1, "f16")
+    want = O.decode_step(q, k, v, kc0, vc0, 0.125, L, acc=np.float64, cache_indir=np.clip(wild, 0, 1), beam_width=2)
+    assert np.abs(got - want).max() <= 1e-3
+
+
+def test_beam_indirection_through_the_extension():
+    """attention_ex(..., cache_indir=, beam_width=) of the PyTorch extension."""
+    from fastforwardattention_amd import FastForwardAttn
+    groups, bw, H, Dh, L = 2, 2, 16, 128, 2100       # 64 pairs x 2100 keys of Dh = 128
+    B = groups * bw
+    rng, K, V, q, k, v = _inputs(9500, B, H, L, Dh, "f16")
+    table = rng.integers(0, bw, (B, L + 1)).astype(np.int32)
+    dev = lambda a: torch.from_numpy(a).to("cuda:0").half()
+    ffa = FastForwardAttn(dev(K), dev(V), L + 1, False)
+    k_cache, v_cache = ffa.get_cache()
+    out = ffa.attention_ex(dev(q), dev(k), dev(v), k_cache, v_cache, 0.1, L, None, 0.0, 0, None, None, None,
+                           cache_indir=torch.from_numpy(table).to("cuda:0"), beam_width=bw)
+    kc0, vc0 = _pack(K, V, L + 1, "f16")
+    want = O.decode_step(q, k, v, kc0, vc0, 0.1, L, acc=np.float64, cache_indir=table, beam_width=bw)
+    assert np.abs(out.float().cpu().numpy() - want).max() <= 1e-3

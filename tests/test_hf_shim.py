@@ -28,17 +28,19 @@ class OracleEngine:
     def get_cache(self):
         return self.kc, self.vc
 
-    def attention(self, q, k, v, k_cache, v_cache, scale, t, *rest):
+    def attention(self, q, k, v, k_cache, v_cache, scale, t, *rest, cache_indir=None, beam_width=1):
         seq_lens, p = (rest[0], rest[1]) if len(rest) == 2 else (None, rest[0])
         assert k_cache is self.kc and v_cache is self.vc and p == 0.0
         shape = (self.B, self.H, self.Dh)
         self.calls.append((t, None if seq_lens is None else seq_lens.tolist(), scale))
         out = O.decode_step(q.detach().numpy().reshape(shape), k.detach().numpy().reshape(shape),
                             v.detach().numpy().reshape(shape), self.kc.numpy(), self.vc.numpy(), scale, t,
-                            seq_lengths=None if seq_lens is None else seq_lens.numpy(), right_or_no_padding=False)
+                            seq_lengths=None if seq_lens is None else seq_lens.numpy(), right_or_no_padding=False,
+                            cache_indir=None if cache_indir is None else cache_indir.numpy(), beam_width=beam_width)
         return torch.from_numpy(out.astype(np.float32))
 
-    def attention_ex(self, q, k, v, k_cache, v_cache, scale, t, seq_lens, p, rotary_dim, q_bias, k_bias, v_bias):
+    def attention_ex(self, q, k, v, k_cache, v_cache, scale, t, seq_lens, p, rotary_dim, q_bias, k_bias, v_bias,
+                     cache_indir=None, beam_width=1):
         """The fused call: the oracle's token transform (rotary embedding at the position
         t - first_key[b]), then the step."""
         assert q_bias is None and k_bias is None and v_bias is None
@@ -50,7 +52,7 @@ class OracleEngine:
         self.rotary_calls = getattr(self, "rotary_calls", []) + [(t, rotary_dim, pos.tolist())]
         rest = (p,) if seq_lens is None else (seq_lens, p)
         return self.attention(torch.from_numpy(q2), torch.from_numpy(k2), torch.from_numpy(v2), k_cache, v_cache,
-                              scale, t, *rest)
+                              scale, t, *rest, cache_indir=cache_indir, beam_width=beam_width)
 
 
 def tiny_opt(dtype=torch.float32):
@@ -138,9 +140,17 @@ def test_cache_refuses_unhooked_model_and_unsupported_operations():
         teacher_forced_logits(model, ids, mask, 1, cache)        # attention never went through the hook
     layer = hf.FFALayer(2, engine=OracleEngine)
     with pytest.raises(NotImplementedError):
-        layer.reorder_cache(torch.tensor([0]))
+        layer.crop(1)
     with pytest.raises(ValueError):
         hf.FFALayer(0)
+    with pytest.raises(ValueError):
+        hf.FFALayer(2, num_beams=0)
+    # beam search with a cache that was not told about the beams: refused, not silently wrong
+    hf.enable(model)
+    kw = dict(attention_mask=mask, max_new_tokens=3, do_sample=False, num_beams=2, pad_token_id=1, eos_token_id=None)
+    with pytest.raises(NotImplementedError, match="num_beams"):
+        model.generate(ids, past_key_values=hf.FFACache(max_new_tokens=3, engine=OracleEngine), **kw)
+    hf.disable(model)
 
 
 def test_env_switches(monkeypatch):
@@ -164,6 +174,57 @@ def test_generate_with_ffa_cache_matches_plain_generate():
     got = model.generate(ids, past_key_values=hf.FFACache(max_new_tokens=5, engine=OracleEngine), **kw)
     hf.disable(model)
     assert torch.equal(got, want)
+
+
+@pytest.mark.parametrize("family", ["opt", "gptj", "gptj_torch_rotary"])
+def test_beam_search_with_ffa_cache_matches_plain_beam_search(family):
+    """generate(num_beams=3): transformers re-parents beams after every step.  Its own cache copies
+    keys and values along the batch axis; the FFACache permutes rows of its table.  Same tokens,
+    and the caches hold exactly what each sample wrote (nothing was moved)."""
+    fused = family != "gptj_torch_rotary"
+    model = tiny_opt() if family == "opt" else tiny_gptj()
+    ids, mask = padded_batch()
+    n, nb = 7, 3
+    kw = dict(attention_mask=mask, max_new_tokens=n, do_sample=False, num_beams=nb, num_return_sequences=nb,
+              pad_token_id=1, eos_token_id=None, length_penalty=0.0)
+    want = model.generate(ids, **kw)
+    hf.enable(model, fused_rotary=fused)
+    cache = hf.FFACache(max_new_tokens=n, engine=OracleEngine, num_beams=nb)
+    got = model.generate(ids, past_key_values=cache, **kw)
+    hf.disable(model)
+    assert torch.equal(got, want)
+    layer = cache.layers[0]
+    table = layer.beam_table.numpy()
+    assert table.shape == (2 * nb, 9 + n) and table.min() >= 0 and table.max() < nb
+    # the search did re-parent: some sample reads a sibling's slots
+    assert (table != (np.arange(2 * nb) % nb)[:, None]).any()
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("family,dtype", [("opt", torch.float32), ("gptj", torch.float32), ("gptj_torch_rotary", torch.float32),
+                                          ("opt", torch.float16), ("gptj", torch.float16)])
+def test_beam_search_with_hip_engine(family, dtype):
+    """Beam search on the GPU through the real extension.  fp32: the same tokens as transformers'
+    own cache.  fp16: sequence scores within 2e-2 (near-ties may order beams differently)."""
+    print("hf beams", family, dtype, flush=True)
+    fused = family != "gptj_torch_rotary"
+    family = family.split("_")[0]
+    model = (tiny_opt(dtype) if family == "opt" else tiny_gptj(dtype)).to("cuda:0")
+    ids, mask = padded_batch("cuda:0")
+    n, nb = 12, 4
+    kw = dict(attention_mask=mask, max_new_tokens=n, do_sample=False, num_beams=nb, num_return_sequences=1,
+              pad_token_id=1, eos_token_id=None, length_penalty=0.0, return_dict_in_generate=True, output_scores=True)
+    want = model.generate(ids, **kw)
+    hf.enable(model, fused_rotary=fused)
+    for use_default in (False, True):
+        cache = hf.FFACache(max_new_tokens=n, num_beams=nb, use_default_kernel_launch=use_default)
+        got = model.generate(ids, past_key_values=cache, **kw)
+        if dtype == torch.float32:
+            assert torch.equal(got.sequences, want.sequences)
+        assert float((got.sequences_scores - want.sequences_scores).abs().max()) < (1e-4 if dtype == torch.float32 else 2e-2)
+        table = cache.layers[0].beam_table.cpu().numpy()
+        assert (table != (np.arange(2 * nb) % nb)[:, None]).any()
+    hf.disable(model)
 
 
 @pytest.mark.gpu

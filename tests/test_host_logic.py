@@ -140,11 +140,13 @@ def test_static_scratch_entry_validates_before_any_launch(lib):
 def test_attention_ex_validates_before_any_launch(lib):
     """ffa_attention_ex: element types, the token transform's fields and the room for the
     transformed token are checked on the host."""
-    def call(precision=16, Dh=64, t=10, rotary=0, q_bias=None, ws=None, ws_bytes=0, plan=None, transform=True):
+    def call(precision=16, Dh=64, t=10, rotary=0, q_bias=None, ws=None, ws_bytes=0, plan=None, transform=True,
+             beams=None):
         tt = capi.TokenTransform(q_bias=q_bias, rotary_embedding_dim=rotary) if transform else None
         return lib.ffa_attention_ex(precision, 2, 4, Dh, 128, 0.125, t, P, P, P, P, P, P, None, 0.0,
                                     C.byref(plan) if plan is not None else None, 1,
-                                    C.byref(tt) if tt is not None else None, ws, ws_bytes, None)
+                                    C.byref(tt) if tt is not None else None,
+                                    C.byref(beams) if beams is not None else None, ws, ws_bytes, None)
     wg = capi.make_plan(capi.FFA_LAUNCH_WORKGROUP, 4, 1, 1)
     assert call(precision=8, plan=wg) == capi.FFA_ERR_DTYPE
     assert call(precision=17, plan=wg) == capi.FFA_ERR_DTYPE
@@ -156,6 +158,15 @@ def test_attention_ex_validates_before_any_launch(lib):
         assert call(precision=prec, rotary=32, plan=wg) == capi.FFA_ERR_WORKSPACE
         assert call(precision=prec, rotary=32, plan=wg, ws=P, ws_bytes=6143) == capi.FFA_ERR_WORKSPACE
     assert "rotary" in capi.status_string(capi.FFA_ERR_TRANSFORM)
+    # beam indirection: batch 2 here
+    BI = capi.BeamIndirection
+    assert call(transform=False, plan=wg, beams=BI(None, 2)) == capi.FFA_ERR_BEAM
+    assert call(transform=False, plan=wg, beams=BI(0x1002, 2)) == capi.FFA_ERR_BEAM      # not 4-byte aligned
+    for bw in (0, -1, 3, 4):
+        assert call(transform=False, plan=wg, beams=BI(0x1000, bw)) == capi.FFA_ERR_BEAM
+    tpk = capi.make_plan(capi.FFA_LAUNCH_SPLIT, 4, 1, 1, threads_per_key=2)
+    assert call(transform=False, plan=tpk, beams=BI(0x1000, 2)) == capi.FFA_ERR_PLAN
+    assert "beam" in capi.status_string(capi.FFA_ERR_BEAM)
     assert lib.ffa_workspace_bytes(2, 4, 64, 128) >= 6144
 
 

@@ -360,3 +360,83 @@ def test_token_transform_invariants():
     np.testing.assert_array_equal(O.rotary_positions(3, 50), [50, 50, 50])
     np.testing.assert_array_equal(O.rotary_positions(3, 50, [10, 50, 0], True), [10, 50, 0])
     np.testing.assert_array_equal(O.rotary_positions(3, 50, [10, 50, 60], False), [40, 0, 0])
+
+
+# ------------------------------------------------------------------ beam-search indirection
+def _beam_problem(seed, groups, bw, H, Dh, L, Lmax, dtype=np.float32):
+    rng = np.random.default_rng(seed)
+    B = groups * bw
+    K = rng.standard_normal((B, H, L, Dh)).astype(dtype)
+    V = rng.standard_normal((B, H, L, Dh)).astype(dtype)
+    return rng, B, O.pack_k_cache(K, Lmax), O.pack_v_cache(V, Lmax)
+
+
+def test_beam_identity_table_is_the_plain_step():
+    groups, bw, H, Dh, L, Lmax = 2, 3, 2, 16, 21, 24
+    rng, B, kc, vc = _beam_problem(70, groups, bw, H, Dh, L, Lmax)
+    q, k, v = (rng.standard_normal((B, H, Dh)).astype(np.float32) for _ in range(3))
+    own = np.repeat((np.arange(B) % bw)[:, None], Lmax, 1).astype(np.int32)
+    kc1, vc1, kc2, vc2 = kc.copy(), vc.copy(), kc.copy(), vc.copy()
+    plain = O.decode_step(q, k, v, kc1, vc1, 0.25, L)
+    beam = O.decode_step(q, k, v, kc2, vc2, 0.25, L, cache_indir=own, beam_width=bw)
+    assert np.array_equal(plain, beam) and np.array_equal(kc1, kc2) and np.array_equal(vc1, vc2)
+    a = O.pruned_decode_step(q, k, v, kc.copy(), vc.copy(), 0.25, L, 1e-2)
+    b = O.pruned_decode_step(q, k, v, kc.copy(), vc.copy(), 0.25, L, 1e-2, cache_indir=own, beam_width=bw)
+    assert all(np.array_equal(x, y) for x, y in zip(a, b))
+
+
+def test_beam_table_reads_follow_the_reference_offsets():
+    """Element by element with the reference's flat offsets (attention.cu:1003, :1027-1031 for
+    K, :1143, :1197-1201 for V): base = group's first beam, plus beam_src whole samples."""
+    groups, bw, H, Dh, L, Lmax = 2, 2, 2, 8, 5, 7
+    rng, B, kc, vc = _beam_problem(71, groups, bw, H, Dh, L, Lmax)
+    x = O.elems_per_16b(np.float32)
+    indir = rng.integers(0, bw, (B, Lmax)).astype(np.int32)
+    kflat, vflat = kc.reshape(-1), vc.reshape(-1)
+    for b in range(B):
+        beami, bbi = b % bw, b // bw
+        Kb, Vb = O.beam_keys_values(kc, vc, b, L + 1, indir, bw)
+        for h in range(H):
+            bbhi = bbi * bw * H + h
+            for ti in range(L):                       # cached keys only: slot L is the new token
+                beam_src = indir.reshape(-1)[(bbi * bw + beami) * Lmax + ti]
+                beam_offset = beam_src * H * Lmax * Dh
+                for d in range(Dh):
+                    ko = bbhi * Lmax * Dh + beam_offset + (d // x) * Lmax * x + ti * x + d % x
+                    vo = bbhi * Lmax * Dh + beam_offset + ti * Dh + d
+                    assert Kb[h, ti, d] == kflat[ko] and Vb[h, ti, d] == vflat[vo]
+            # the new token's slot is the sample's own
+            assert np.array_equal(Kb[h, L], O.unpack_k_cache(kc[b:b + 1], L + 1)[0, h, L])
+            assert np.array_equal(Vb[h, L], vc[b, h, L])
+
+
+@pytest.mark.parametrize("p", [0.0, 2e-2])
+def test_beam_search_by_table_equals_beam_search_by_cache_copy(p):
+    """A toy beam search, two ways.  By copy: after every step the caches of each group are
+    re-gathered by the chosen parents, as the reference's models do
+    (_reorder_cache = index_select on the batch axis, modeling_opt.py:1072-1075), and the step
+    reads a sample's own caches.  By table: caches stay where they were written; the table row
+    of a beam becomes its parent's row, and the token a beam has just written is its own.
+    Outputs must agree bit for bit at every step."""
+    groups, bw, H, Dh, L, steps = 2, 3, 2, 16, 9, 7
+    Lmax = L + steps
+    rng, B, kc, vc = _beam_problem(72, groups, bw, H, Dh, L, Lmax)
+    kc_copy, vc_copy = kc.copy(), vc.copy()
+    table = np.repeat((np.arange(B) % bw)[:, None], Lmax, 1).astype(np.int32)
+    for s in range(steps):
+        t = L + s
+        q, k, v = (rng.standard_normal((B, H, Dh)).astype(np.float32) for _ in range(3))
+        if p == 0.0:
+            by_copy = O.decode_step(q, k, v, kc_copy, vc_copy, 0.25, t)
+            by_table = O.decode_step(q, k, v, kc, vc, 0.25, t, cache_indir=table, beam_width=bw)
+        else:
+            by_copy = O.pruned_decode_step(q, k, v, kc_copy, vc_copy, 0.25, t, p)[0]
+            by_table = O.pruned_decode_step(q, k, v, kc, vc, 0.25, t, p, cache_indir=table, beam_width=bw)[0]
+        assert np.array_equal(by_copy, by_table), s
+        # every beam picks a parent inside its group
+        parent = (np.arange(B) // bw) * bw + rng.integers(0, bw, B)
+        kc_copy, vc_copy = kc_copy[parent].copy(), vc_copy[parent].copy()
+        new_table = table[parent].copy()
+        new_table[:, t] = parent % bw                 # slot t was written by the parent itself
+        table = new_table
+    assert len(np.unique(table[:, :Lmax - 1], axis=0)) > groups   # the search did mix beams
