@@ -81,6 +81,25 @@ __device__ __forceinline__ void step_bounds(const DecodeParams& P, int b, int& t
     }
 }
 
+// Order in which a workgroup walks its tiles [lo, hi): rotated by an offset that differs from
+// workgroup to workgroup.  All workgroups of a launch run the same loop at the same pace over
+// caches a fixed stride apart, so without the rotation their loads fall on the same memory
+// channels at the same time whenever that stride folds badly onto the channel map (measured:
+// 512 pairs x 8192 keys with rows of 8256 slots 166 -> 155 us for the loads alone, rows of
+// 2048 slots at 1000 keys 20.0 -> 18.0 us; nothing lost at strides that were good already).
+// The result does not depend on the order beyond the rounding of the running sums.
+struct TileOrder {
+    int lo, n, rot;
+    __device__ __forceinline__ TileOrder(int lo_, int hi_, unsigned salt) : lo(lo_), n(max(hi_ - lo_, 0)), rot(0) {
+        if (n > 1) rot = (int)(((salt * 2654435761u) >> 8) % (unsigned)n);
+    }
+    // Tile at position idx of the walk, idx in [0, n).
+    __device__ __forceinline__ int at(int idx) const {
+        const int a = idx + rot;
+        return lo + (a >= n ? a - n : a);
+    }
+};
+
 // Append k_new, v_new at slot tlen of the (b,h) caches (attention.cu:901-914, :1246).
 // One wave: lane c < NCH moves 16-byte chunk c of K and of V (NCH <= 64).  The loads are
 // issued early (new_token_load) and the stores late (new_token_store), so that neither
@@ -573,10 +592,12 @@ __global__ void __launch_bounds__(NW * 64) ffa_decode_split_kernel(const DecodeP
     // save registers, which would serialise the round trips.  With beam indirection the
     // source beams of a tile are fetched one tile ahead, so that their round trip does not sit
     // in front of the tile's own loads.
-    int src_next = beams.beam((tile_lo + wave) * kWave + lane, tlen);
-    for (int tile = tile_lo + wave; tile < tile_hi; tile += NW) {
+    const TileOrder order(tile_lo, tile_hi, (unsigned)(bh * n_splits + split));
+    int src_next = beams.beam(order.at(wave) * kWave + lane, wave < order.n ? tlen : 0);
+    for (int idx = wave; idx < order.n; idx += NW) {
+        const int tile = order.at(idx);
         const int src = src_next;
-        if constexpr (BEAM) src_next = beams.beam((tile + NW) * kWave + lane, tile + NW < tile_hi ? tlen : 0);
+        if constexpr (BEAM) src_next = beams.beam(order.at(idx + NW) * kWave + lane, idx + NW < order.n ? tlen : 0);
         uint4 kv[CG], vv[VG];
         load_tile(kv, vv, tile, src);
         __builtin_amdgcn_sched_barrier(0);
@@ -655,7 +676,9 @@ __global__ void __launch_bounds__(NW * 64) ffa_decode_split_tpk_kernel(const Dec
 #pragma unroll
     for (int e = 0; e < X; ++e) acc[e] = 0.f;
 
-    for (int tile = tile_lo + wave; tile < tile_hi; tile += NW) {
+    const TileOrder order(tile_lo, tile_hi, (unsigned)(bh * n_splits + split));
+    for (int idx = wave; idx < order.n; idx += NW) {
+        const int tile = order.at(idx);
         const int key = tile * KPT + kl;
         const bool cached = key < tlen;
         const char* kp = cached ? kc_bh + ((size_t)(part * NK) * P.Lmax + key) * 16 : knew + part * NK * 16;
@@ -773,7 +796,9 @@ __global__ void __launch_bounds__(NW * 64) ffa_decode_wg_kernel(const DecodePara
 
     // ---- phase 1: raw scores to LDS, running max (exp2 domain) ----
     float mx = -INFINITY;
-    for (int tile = tile_lo + wave; tile < ntiles; tile += NW) {
+    const TileOrder order(tile_lo, ntiles, (unsigned)bh);
+    for (int idx = wave; idx < order.n; idx += NW) {
+        const int tile = order.at(idx);
         const int key = tile * kWave + lane;
         float s = tile_qk<T, NCH, G::Q_LDS>(beams.k_of(beams.beam(key, tlen)), knew, key, tlen, P.Lmax, q_reg, s_q);
         const bool valid = key <= tlen && key >= first;
@@ -859,7 +884,8 @@ __global__ void __launch_bounds__(NW * 64) ffa_decode_wg_kernel(const DecodePara
     for (int e = 0; e < X; ++e) acc[e] = 0.f;
     if (pruned) {
         SurvivorQueue sq = {s_qw[wave], s_qr[wave], 0u};
-        for (int tile = tile_lo + wave; tile < ntiles; tile += NW) {
+        for (int idx = wave; idx < order.n; idx += NW) {
+            const int tile = order.at(idx);
             const int key = tile * kWave + lane;
             const float w = s_sc[key];
             const int row = beams.v_row(beams.beam(key, tlen), key, tlen, rows_per_sample);
@@ -867,7 +893,8 @@ __global__ void __launch_bounds__(NW * 64) ffa_decode_wg_kernel(const DecodePara
         }
         queue_drain<T, DH>(acc, sq, beams.v_group, vnew, lane);
     } else {
-        for (int tile = tile_lo + wave; tile < ntiles; tile += NW) {
+        for (int idx = wave; idx < order.n; idx += NW) {
+            const int tile = order.at(idx);
             const int src = beams.beam(tile * kWave + lane, tlen);  // a row's beam sits in its key's lane
 #pragma unroll 1
             for (int g = 0; g < NVL / VG; ++g) {
@@ -957,7 +984,9 @@ __global__ void __launch_bounds__(NW * 64) ffa_scores_kernel(const DecodeParams 
     const BeamRows<BEAM> beams(P, b, bh, head_bytes);
     float* sc = P.ws_scores + (size_t)bh * P.score_stride;
     float m_run = -INFINITY, l_run = 0.f;
-    for (int tile = tile_lo + wave; tile < tile_hi; tile += NW) {
+    const TileOrder order(tile_lo, tile_hi, (unsigned)blockIdx.x);
+    for (int idx = wave; idx < order.n; idx += NW) {
+        const int tile = order.at(idx);
         const int key = tile * kWave + lane;
         const float s = tile_qk<T, NCH, G::Q_LDS>(beams.k_of(beams.beam(key, tlen)), knew, key, tlen, P.Lmax, q_reg, s_q);
         const bool valid = key <= tlen && key >= first;
@@ -1023,8 +1052,9 @@ __global__ void __launch_bounds__(NW * 64) ffa_pruned_pv_kernel(const DecodePara
     // folds them through the same reduction tree, so all arrive at bit-identical M, S ----
     static_assert(kMaxSplits <= 2 * kWave, "two pieces per lane at most");
     // The first tile's scores (and source beams) travel together with the pieces' (max, sum).
-    float sr_next = (tile_lo + wave < tile_hi) ? sc[(tile_lo + wave) * kWave + lane] : -INFINITY;
-    int src_next = beams.beam((tile_lo + wave) * kWave + lane, tile_lo + wave < tile_hi ? tlen : 0);
+    const TileOrder order(tile_lo, tile_hi, (unsigned)blockIdx.x);
+    float sr_next = (wave < order.n) ? sc[order.at(wave) * kWave + lane] : -INFINITY;
+    int src_next = beams.beam(order.at(wave) * kWave + lane, wave < order.n ? tlen : 0);
     const float* ml = P.ws_ml + (size_t)bh * P.n_splits * 2;
     float m_a = -INFINITY, l_a = 0.f, m_b = -INFINITY, l_b = 0.f;
     if (lane < P.n_splits) {
@@ -1053,12 +1083,13 @@ __global__ void __launch_bounds__(NW * 64) ffa_pruned_pv_kernel(const DecodePara
     for (int e = 0; e < X; ++e) acc[e] = 0.f;
     unsigned kept = 0;
     SurvivorQueue sq = {s_qw[wave], s_qr[wave], 0u};
-    for (int tile = tile_lo + wave; tile < tile_hi; tile += NW) {
-        const int key = tile * kWave + lane;
+    for (int idx = wave; idx < order.n; idx += NW) {
+        const int key = order.at(idx) * kWave + lane;
         const float sr = sr_next;
         const int src = src_next;
-        sr_next = (tile + NW < tile_hi) ? sc[key + NW * kWave] : -INFINITY;  // one tile ahead
-        src_next = beams.beam(key + NW * kWave, tile + NW < tile_hi ? tlen : 0);
+        const int key_next = order.at(idx + NW) * kWave + lane;  // one tile ahead
+        sr_next = (idx + NW < order.n) ? sc[key_next] : -INFINITY;
+        src_next = beams.beam(key_next, idx + NW < order.n ? tlen : 0);
         const float e = (sr == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(fmaf(sr, P.scale_log2e, -M));
         const bool in_range = key >= first && key <= tlen;
         float w;
