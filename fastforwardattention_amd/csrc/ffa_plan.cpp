@@ -158,10 +158,10 @@ static int plan_by_rules(int precision, int B, int H, int Dh, int t, float p, in
     //  - Fewer pairs than CUs: floor(CUs/pairs) pieces per pair (one workgroup per CU), but
     //    never so many that a wave is left without a tile.
     //  - Long sequences with at least one pair per CU: the one-workgroup kernel with 16 waves
-    //    (70 VGPRs, two workgroups = 32 waves resident per CU, separate K and V phases) streams
-    //    up to 8 % faster than the split kernel (8192 keys: 256 pairs 91 vs 99 us, 512 pairs
-    //    181 vs 193 us, 1024 pairs 353 vs 373 us; 4096 keys: 84 vs 85, 167 vs 170 us); below
-    //    4096 keys the split kernel is ahead.
+    //    (separate K and V phases).  Every exact launch is within 1 % of the others there
+    //    (512 pairs x 8192 keys: 163 to 166 us for the split kernel with 4 or 8 waves and this
+    //    kernel with 4, 8 or 16 waves); this one also serves the pruned steps of such shapes.
+    //    Below 4096 keys the split kernel is ahead.
     if (bh >= cus && ntiles >= 64 && fits_wg) {
         fill(plan, FFA_LAUNCH_WORKGROUP, 16, 1, ntiles);
         return FFA_OK;
