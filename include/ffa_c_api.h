@@ -202,8 +202,9 @@ int ffa_attention_diag(int precision, int batch_size, int head_num, int head_dim
  *              the step and in this order: q += q_bias, k += k_bias, v += v_bias (device
  *              [H, Dh] arrays of the element type, each may be NULL); then, if
  *              rotary_embedding_dim > 0 (even, <= head_dim), the pairs (2i, 2i+1) below that
- *              dimension of q and k are rotated by pos / base^(2i / rotary_embedding_dim),
- *              computed in fp32 and rounded once (GPT-J's convention).  pos is the number of
+ *              dimension of q and k are rotated by pos / base^(2i / rotary_embedding_dim)
+ *              (GPT-J's pairing), evaluated in double precision and rounded once to the
+ *              element type.  pos is the number of
  *              real tokens before the new one: t, or seq_lengths[b] with right padding, or
  *              t - seq_lengths[b] with left padding (the reference rotates by t alone and so
  *              supports no padded batch, attention.cu:879).  The transformed k and v are what
