@@ -342,7 +342,36 @@ def cpu_baseline(wl, budget_s=12.0, max_steps=40000):
                    f"{', repeated' if len(times) > span * nlayers else ''}; {sum(times):.1f} s of CPU work), "
                    "fp32 torch bmm/softmax/bmm over a pre-allocated cache; bytes counted at 4 B/element"),
         "config1": cpu_baseline_config1(),
+        "small_batches": cpu_baseline_small_batches(wl),
     }
+
+
+def cpu_baseline_small_batches(wl, budget_s=1.5):
+    """The same CPU decode loop at the workload's shape with B = 1, 2, 5 (the other batch sizes of
+    BASELINE configs[1]): at least 16 steps each, about `budget_s` seconds of CPU work per batch."""
+    import torch
+    from oracle.torch_attn import CpuDecodeBaseline
+    H, Dh, L = wl.H, wl.Dh, wl.prompt
+    out = []
+    for B in (1, 2, 5):
+        g = torch.Generator().manual_seed(B)
+        base = CpuDecodeBaseline(torch.randn(B, H, L, Dh, generator=g) * 0.5, torch.randn(B, H, L, Dh, generator=g) * 0.5,
+                                 wl.Lmax)
+        toks = [tuple(torch.randn(B, H, Dh, generator=g) for _ in range(3)) for _ in range(4)]
+        span = max(1, wl.gen - 4)
+        for i in range(3):
+            base.attention(*toks[i % 4], wl.scale, L + i)
+        times, t0 = [], time.perf_counter()
+        while len(times) < 16 or (time.perf_counter() - t0 < budget_s and len(times) < 20000):
+            s = time.perf_counter()
+            base.attention(*toks[len(times) % 4], wl.scale, L + 3 + len(times) % span)
+            times.append(time.perf_counter() - s)
+        mean_s = sum(times) / len(times)
+        t_mid = L + 3 + (min(len(times), span) - 1) // 2
+        out.append({"B": B, "us_per_step": round(mean_s * 1e6, 1), "steps": len(times),
+                    "GBps": round(algorithmic_bytes(B, H, Dh, t_mid, elem=4) / mean_s / 1e9, 2),
+                    "threads": torch.get_num_threads()})
+    return out
 
 
 def cpu_baseline_config1(budget_s=2.0):
