@@ -1,6 +1,7 @@
 """GPU parity at the BASELINE shapes themselves, through the C ABI, against the CPU oracle:
 the long-sequence sweep (B=1, 32x64, up to 16384 keys) with both launches, the pruned sweep
 (B=16, 32x64, 8192 keys, peaked keys, four thresholds), the OPT-1.3b shape at B=1 and B=5,
+the GPT-J shape (B=8, 16x256, 2000 to 2255 keys),
 and the one-workgroup kernel in the range where its scores need more than 48 KiB of LDS.
 Tolerances: 1e-3 max-abs for fp16 inputs, 1e-6 for fp32 inputs, against the float64 closed
 form; caches bit for bit; skip sets equal to the rule's except within one quantum of the
@@ -81,6 +82,39 @@ def test_opt13b_shape_small_batches(B):
         gk, gv = sess.caches()
         np.testing.assert_array_equal(gk.view(np.uint8), kc.view(np.uint8))
         np.testing.assert_array_equal(gv.view(np.uint8), vc.view(np.uint8))
+
+
+# ------------------------------------------------------------------ configs[3]: GPT-J shape
+@pytest.mark.parametrize("t0", [2000, 2060, 2250])
+def test_gptj_shape_steps(t0):
+    """BASELINE configs[3]: B=8, 16 heads x 256, fp16, prompt 2000, max_len 2256.  Steps around
+    t0 with the launch the library plans (one lane per key below 2065 keys, four lanes per key
+    from there on: the planner's measured table) and the default launch, against the oracle;
+    caches bit for bit."""
+    B, H, Dh, prec, Lmax, steps = 8, 16, 256, 16, 2256, 6
+    rng, K, V = rand_inputs(500 + t0, B, H, t0, Dh, prec, kv_scale=0.5)
+    scale = 1.0 / 16.0
+    kinds = set()
+    for use_default in (False, True):
+        sess = CApiSession(K, V, Lmax)
+        kc, vc = O.pack_k_cache(K, Lmax), O.pack_v_cache(V, Lmax)
+        worst = 0.0
+        for i in range(steps):
+            t = t0 + i
+            q, k, v = rand_token(rng, B, H, Dh, prec)
+            plan = capi.plan_launch(prec, B, H, Dh, t, 0.0, use_default)
+            kinds.add((plan.kind, plan.threads_per_key))
+            _say("gptj", use_default, t, plan)
+            got = sess.step(q, k, v, scale, t, plan=plan)
+            want = O.decode_step(q, k, v, kc, vc, scale, t, acc=np.float64)
+            worst = max(worst, float(np.abs(got - want).max()))
+        assert worst <= TOL[prec], worst
+        gk, gv = sess.caches()
+        n = t0 + steps                       # slots beyond are untouched (and unspecified) on both sides
+        np.testing.assert_array_equal(gk[:, :, :, :n].view(np.uint16), kc[:, :, :, :n].view(np.uint16))
+        np.testing.assert_array_equal(gv[:, :, :n].view(np.uint16), vc[:, :, :n].view(np.uint16))
+    if t0 == 2060:      # the steps cross from one lane per key to four
+        assert (capi.FFA_LAUNCH_SPLIT, 1) in kinds and (capi.FFA_LAUNCH_SPLIT, 4) in kinds
 
 
 # ------------------------------------------------------------------ configs[4]: pruned sweep, B = 16
