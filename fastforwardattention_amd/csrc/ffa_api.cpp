@@ -61,26 +61,28 @@ int run_decode(const DecodeArgs& args, const ffa_launch_plan* user_plan, void* w
     if (diag && plan.kind == FFA_LAUNCH_SPLIT) return FFA_ERR_PLAN;
     if (a.cache_indir != nullptr && plan.threads_per_key > 1) return FFA_ERR_PLAN;
 
+    // Workspace layout: [arrival counters][transformed token (only with a transform)][what the
+    // plan needs].  The counters are the only words that persist from call to call, so nothing
+    // else may ever be placed on them, whatever the plan of this step or of an earlier one is.
     WorkspaceView ws = {nullptr, nullptr, nullptr, nullptr, 0};
     const int bh = a.B * a.H;
     const int split_heads = bh - plan.whole_heads;
-    if (a.transforms_token()) {
-        // The transformed q, k, v sit behind what the plan itself uses of the workspace.
-        const size_t plan_bytes = align_up(plan_workspace_bytes(plan, bh, a.Dh, a.Lmax), 256);
-        if (workspace == nullptr || workspace_bytes < plan_bytes + token_scratch_bytes(bh, a.Dh))
-            return FFA_ERR_WORKSPACE;
+    const size_t need = decode_workspace_bytes(plan, bh, a.Dh, a.Lmax, a.transforms_token());
+    if (need > 0) {
+        if (workspace == nullptr || workspace_bytes < need) return FFA_ERR_WORKSPACE;
         if (!aligned16(workspace)) return FFA_ERR_ALIGNMENT;
-        a.token_scratch = static_cast<char*>(workspace) + plan_bytes;
     }
-    if (plan.kind == FFA_LAUNCH_TWO_PASS) {
-        // [counters][piece (max, sum)][partial outputs][scores]
-        if (workspace == nullptr ||
-            workspace_bytes < two_pass_workspace_bytes(bh, a.Dh, plan.n_splits, a.Lmax))
-            return FFA_ERR_WORKSPACE;
-        if (!aligned16(workspace)) return FFA_ERR_ALIGNMENT;
-        char* base = static_cast<char*>(workspace);
+    char* base = static_cast<char*>(workspace);
+    if (need > 0) {
         ws.cnt = reinterpret_cast<unsigned int*>(base);
         base += workspace_counter_bytes(bh);
+    }
+    if (a.transforms_token()) {
+        a.token_scratch = base;
+        base += token_scratch_bytes(bh, a.Dh);
+    }
+    if (plan.kind == FFA_LAUNCH_TWO_PASS) {
+        // [piece (max, sum)][partial outputs][scores]
         ws.ml = reinterpret_cast<float*>(base);
         base += align_up((size_t)bh * plan.n_splits * 2 * sizeof(float), 256);
         ws.acc = reinterpret_cast<float*>(base);
@@ -88,16 +90,9 @@ int run_decode(const DecodeArgs& args, const ffa_launch_plan* user_plan, void* w
         ws.scores = reinterpret_cast<float*>(base);
         ws.score_stride = score_stride_for(a.Lmax);
     } else if (plan.kind == FFA_LAUNCH_SPLIT && plan.n_splits > 1 && split_heads > 0) {
-        if (workspace == nullptr ||
-            workspace_bytes < workspace_bytes_for(bh, split_heads, a.Dh, plan.n_splits))
-            return FFA_ERR_WORKSPACE;
-        if (!aligned16(workspace)) return FFA_ERR_ALIGNMENT;
-        char* base = static_cast<char*>(workspace);
-        ws.cnt = reinterpret_cast<unsigned int*>(base);
-        ws.ml = reinterpret_cast<float*>(base + workspace_counter_bytes(bh));
+        ws.ml = reinterpret_cast<float*>(base);
         ws.acc = reinterpret_cast<float*>(
-            base + workspace_counter_bytes(bh) +
-            align_up((size_t)split_heads * plan.n_splits * 2 * sizeof(float), 256));
+            base + align_up((size_t)split_heads * plan.n_splits * 2 * sizeof(float), 256));
     }
     return launch_decode(a, plan, ws);
 }
@@ -150,7 +145,7 @@ static int plan_entry(int precision, int batch_size, int head_num, int head_dim,
         compute_units = query_compute_units();
         if (compute_units <= 0) return FFA_ERR_NO_DEVICE;
     }
-    return plan_launch_ex(precision, batch_size, head_num, head_dim, t, prob_thresh,
+    return plan_launch_ex(planner_precision(precision), batch_size, head_num, head_dim, t, prob_thresh,
                           use_default_kernel_launch, compute_units, use_table, plan);
 }
 
@@ -180,12 +175,11 @@ size_t ffa_workspace_bytes(int batch_size, int head_num, int head_dim, int max_s
 int ffa_workspace_init(void* workspace, size_t workspace_bytes, void* stream) {
     if (workspace == nullptr) return FFA_ERR_NULL_POINTER;
     if (!aligned16(workspace)) return FFA_ERR_ALIGNMENT;
-    // Only the arrival counters at the head of the workspace have to start at zero; every
-    // other word is written before it is read.  A workspace of ffa_workspace_bytes() holds at
-    // least 268 bytes per (batch, head) pair (4 of counter, 8 + 4*Dh of partials, Dh >= 64),
-    // so the counter block lies within its first 64th (plus the block's 256-byte alignment).
-    size_t bytes = align_up(workspace_bytes / 64, 256) + 256;
-    if (bytes > workspace_bytes) bytes = workspace_bytes;
+    // Only the arrival counters at the head of the workspace have to start at zero, but how many
+    // there are depends on the problem (4 bytes per (batch, head) pair), which this call does not
+    // know, and a caller may hand over a buffer sized for one plan rather than
+    // ffa_workspace_bytes().  The call is made once per workspace: clear all of it.
+    const size_t bytes = workspace_bytes & ~(size_t)3;
     return launch_fill_u32(static_cast<unsigned int*>(workspace), bytes / 4, 0u, stream);
 }
 

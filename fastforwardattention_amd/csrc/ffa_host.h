@@ -109,6 +109,15 @@ inline size_t plan_workspace_bytes(const ffa_launch_plan& plan, int bh, int head
     return 0;
 }
 
+// Bytes of workspace one decode call touches: the counter block always leads, the transformed
+// token (if any) follows it, the plan's own regions come last.
+inline size_t decode_workspace_bytes(const ffa_launch_plan& plan, int bh, int head_dim, int max_seq_len,
+                                     bool transforms_token) {
+    const size_t plan_bytes = plan_workspace_bytes(plan, bh, head_dim, max_seq_len);
+    if (!transforms_token) return plan_bytes;
+    return (plan_bytes > 0 ? plan_bytes : workspace_counter_bytes(bh)) + token_scratch_bytes(bh, head_dim);
+}
+
 // Size of the library's own scratch array (one per GPU, held until the process ends), used by
 // ffa_attention_static_scratch in place of a caller-owned workspace.
 constexpr size_t kStaticScratchBytes = FFA_STATIC_SCRATCH_BYTES;

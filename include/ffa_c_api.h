@@ -58,8 +58,10 @@ typedef enum ffa_status {
  * (torch_ffa_api.cpp:174). */
 #define FFA_PRECISION_F16 16
 #define FFA_PRECISION_F32 32
-/* bfloat16 (1-8-7), accepted by ffa_attention_ex only.  The reference carries a bf16 build
- * (ENABLE_BF16, decoder_masked_multihead_attention_utils.h:44-125) that it never enables. */
+/* bfloat16 (1-8-7), accepted by ffa_attention_ex, ffa_attention_diag and
+ * ffa_attention_static_scratch (and by the planner, which plans it like fp16).  The reference
+ * carries a bf16 build (ENABLE_BF16, decoder_masked_multihead_attention_utils.h:44-125) that it
+ * never enables. */
 #define FFA_PRECISION_BF16 0xBF16
 
 /* Launch kinds. */
@@ -126,8 +128,8 @@ int ffa_plan_launch_rules(int precision, int batch_size, int head_num, int head_
  * of ffa_attention_ex). */
 size_t ffa_workspace_bytes(int batch_size, int head_num, int head_dim, int max_seq_len);
 
-/* Zero the arrival counters of a workspace of ffa_workspace_bytes() bytes (they sit at its
- * head; the rest is left as it is).  Call once before first use, and again after any launch
+/* Zero a workspace (what matters are the arrival counters at its head; the buffer may be of
+ * ffa_workspace_bytes() bytes or sized for one plan).  Call once before first use, and again after any launch
  * on the workspace that failed or was aborted: a launch that dies half-way leaves counters
  * non-zero, and later launches would then never merge their pieces.
  * One workspace serves one stream at a time: two launches that overlap on the same

@@ -444,3 +444,96 @@ def test_beam_indirection_through_the_extension():
     kc0, vc0 = _pack(K, V, L + 1, "f16")
     want = O.decode_step(q, k, v, kc0, vc0, 0.1, L, acc=np.float64, cache_indir=table, beam_width=bw)
     assert np.abs(out.float().cpu().numpy() - want).max() <= 1e-3
+
+
+# ------------------------------------------------------------------ one workspace, changing plans
+def _transform_step_check(sess, rng, kc, vc, t, elem, rd, biases, scale, p=0.0, plan=None, tag=""):
+    """One ffa_attention_ex step with a transform on a long-lived session, against the oracle
+    (which appends to kc, vc).  Returns the worst output error."""
+    B, H, Dh = sess.B, sess.H, sess.Dh
+    q, k, v = (O.round_to(rng.standard_normal((B, H, Dh)), elem) for _ in range(3))
+    pos = O.rotary_positions(B, t)
+    q2, k2, v2 = O.token_transform(q, k, v, elem, biases.get("q_bias"), biases.get("k_bias"), biases.get("v_bias"), rd, pos)
+    want = O.decode_step(q2, k2, v2, kc, vc, scale, t, acc=np.float64)
+    got = sess.step(q, k, v, scale, t, p=p, plan=plan, transform=dict(biases, rotary_dim=rd))
+    assert np.isfinite(got).all(), (tag, t, "output was never written")
+    err = float(np.abs(got - want).max())
+    assert err <= {"f16": 1e-3 + 3e-4, "f32": 2e-6}[elem], (tag, t, err)
+    return err
+
+
+def _check_caches_after_transforms(sess, kc, vc, n, elem):
+    gk, gv = _cache_values(sess)
+    dk = np.abs(gk[:, :, :, :n] - kc[:, :, :, :n])
+    assert (dk <= _ulp(kc[:, :, :, :n], elem) * 1.01).all() and (dk != 0).mean() < 0.01
+    np.testing.assert_array_equal(gv[:, :, :n], vc[:, :, :n])
+
+
+def test_rotary_decode_on_one_workspace_across_plan_changes():
+    """GPT-J-shaped iterative decode at B = 1 (16 heads x 256, rotary_dim 64, fp16), t = 100 -> 300,
+    ONE session and ONE workspace, the library's own plan at every step.  The planner moves between
+    launches that use no workspace and sequence-split launches on the way (the test asserts that
+    it does), so whatever a step leaves in the workspace meets the arrival counters of a later
+    step.  Reference: the token transform of attention.cu:856-882 keeps no state between calls."""
+    B, H, Dh, L, rd, elem, end = 1, 16, 256, 100, 64, "f16", 300
+    rng, K, V, *_ = _inputs(4100, B, H, L, Dh, elem)
+    sess = ExSession(K, V, end + 1, elem)
+    kc, vc = _pack(K, V, end + 1, elem)
+    kinds = set()
+    for t in range(L, end):
+        plan = capi.plan_launch(16, B, H, Dh, t, 0.0, False, sess.lib.ffa_device_compute_units())
+        kinds.add((plan.kind, plan.n_splits > 1))
+        _transform_step_check(sess, rng, kc, vc, t, elem, rd, {}, 1.0 / 16, tag=repr(plan))
+    assert any(s for _, s in kinds) and any(not s for _, s in kinds), kinds   # both sides of the switch were run
+    _check_caches_after_transforms(sess, kc, vc, end, elem)
+
+
+@pytest.mark.parametrize("elem", ["f16", "f32"])
+def test_transform_steps_of_every_launch_kind_share_one_workspace(elem):
+    """Bias + rotary steps on one workspace in the order that used to break: a one-workgroup launch
+    (needs no workspace of its own), a sequence-split launch with a fused merge, a pruned two-pass
+    launch, a split launch merged by a second kernel, and round again."""
+    B, H, Dh, L, rd = 2, 3, 64, 700, 32
+    rng, K, V, *_ = _inputs(4200, B, H, L, Dh, elem)
+    steps = 10
+    sess = ExSession(K, V, L + steps, elem)
+    kc, vc = _pack(K, V, L + steps, elem)
+    biases = {n: O.round_to(rng.standard_normal((H, Dh)), elem) for n in ("q_bias", "k_bias", "v_bias")}
+    for i in range(steps):
+        t = L + i
+        ntiles = t // 64 + 1
+        plan, p = [
+            (capi.make_plan(capi.FFA_LAUNCH_WORKGROUP, 4, 1, ntiles), 0.0),
+            (capi.make_plan(capi.FFA_LAUNCH_SPLIT, 4, -(-ntiles // 3), 3), 0.0),
+            (capi.make_plan(capi.FFA_LAUNCH_TWO_PASS, 4, -(-ntiles // 2), 2), 1e-7),   # below every probability
+            (capi.make_plan(capi.FFA_LAUNCH_SPLIT, 2, -(-ntiles // 4), 4, capi.FFA_COMBINE_KERNEL), 0.0),
+            (capi.make_plan(capi.FFA_LAUNCH_SPLIT, 4, 1, ntiles, whole_heads=B * H), 0.0),
+        ][i % 5]
+        _say("shared workspace", elem, i, plan)
+        _transform_step_check(sess, rng, kc, vc, t, elem, rd, biases, 0.125, p=p, plan=plan, tag=repr(plan))
+    _check_caches_after_transforms(sess, kc, vc, L + steps, elem)
+
+
+def test_alternating_pruned_and_exact_calls_on_one_object():
+    """attention_ex of the Python class with the rotary embedding, p > 0 and p = 0 in turn: at this
+    shape a pruned step is a one-workgroup launch and an exact step a sequence-split one, on the
+    object's one workspace."""
+    from fastforwardattention_amd import FastForwardAttn
+    B, H, Dh, L, rd, steps = 4, 32, 64, 300, 32, 12
+    rng, K, V, *_ = _inputs(4300, B, H, L, Dh, "f16")
+    dev = lambda a: torch.from_numpy(np.ascontiguousarray(a, np.float32)).to("cuda:0").half()
+    ffa = FastForwardAttn(dev(K), dev(V), L + steps, False)
+    k_cache, v_cache = ffa.get_cache()
+    kc, vc = _pack(K, V, L + steps, "f16")
+    plans = set()
+    for i in range(steps):
+        t, p = L + i, (1e-7 if i % 2 == 0 else 0.0)
+        plans.add(tuple(ffa.launch_plan(t, p))[:1] + (tuple(ffa.launch_plan(t, p))[4] > 1,))
+        q, k, v = (O.round_to(rng.standard_normal((B, H, Dh)), "f16") for _ in range(3))
+        q2, k2, v2 = O.token_transform(q, k, v, "f16", rotary_dim=rd, pos=O.rotary_positions(B, t))
+        want = O.decode_step(q2, k2, v2, kc, vc, 0.125, t, acc=np.float64)
+        out = ffa.attention_ex(dev(q), dev(k), dev(v), k_cache, v_cache, 0.125, t, None, p, rd, None, None, None)
+        got = out.float().cpu().numpy()
+        assert np.isfinite(got).all(), i
+        assert np.abs(got - want).max() <= 1e-3 + 3e-4, (i, p)
+    assert (capi.FFA_LAUNCH_WORKGROUP, False) in plans and (capi.FFA_LAUNCH_SPLIT, True) in plans, plans

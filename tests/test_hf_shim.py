@@ -86,7 +86,7 @@ def teacher_forced_logits(model, ids, mask, steps, cache):
         logits.append(out.logits[:, -1].float())
         cache = out.past_key_values
         for i in range(steps):
-            tok = torch.full((ids.shape[0], 1), 30 + i, device=ids.device, dtype=ids.dtype)
+            tok = torch.full((ids.shape[0], 1), 30 + i % 60, device=ids.device, dtype=ids.dtype)   # stays inside the 96-token vocabulary
             mask = torch.cat([mask, torch.ones_like(mask[:, :1])], dim=1)
             pos = (mask.long().cumsum(-1) - 1)[:, -1:]
             kw = {"position_ids": pos} if "GPTJ" in type(model).__name__ else {}
@@ -255,3 +255,35 @@ def test_hook_with_hip_engine(family, dtype, tol):
     got, _ = teacher_forced_logits(model, ids, mask, steps, hf.FFACache(max_new_tokens=steps, prob_thresh=1e-7))
     assert float((got - want).abs().max()) < tol
     hf.disable(model)
+
+
+def small_gptj(dtype=torch.float32):
+    """Four heads of 64, room for 256 positions: long enough for the launch plan of a decode to
+    move from one workgroup per head to sequence-split launches."""
+    cfg = transformers.GPTJConfig(vocab_size=96, n_positions=256, n_embd=256, n_layer=2, n_head=4, rotary_dim=32,
+                                  n_inner=256, resid_pdrop=0.0, embd_pdrop=0.0, attn_pdrop=0.0,
+                                  bos_token_id=2, eos_token_id=2)
+    torch.manual_seed(0)
+    return transformers.GPTJForCausalLM(cfg).to(dtype).eval()
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype,tol", [(torch.float32, 2e-4), (torch.float16, 3e-2)])
+def test_long_decode_with_fused_rotary_crosses_launch_plans(dtype, tol):
+    """170 decode steps from a 9-token prompt through the hook with the rotary embedding inside the
+    engine's call, one engine (one workspace) per layer for the whole decode; the logits of every
+    step against transformers' own cache.  The engine's plan changes kind on the way."""
+    print("hf long decode", dtype, flush=True)
+    model = small_gptj(dtype).to("cuda:0")
+    ids, mask = padded_batch("cuda:0")
+    steps = 170
+    want, _ = teacher_forced_logits(model, ids, mask, steps, None)
+    hf.enable(model, fused_rotary=True)
+    got, cache = teacher_forced_logits(model, ids, mask, steps, hf.FFACache(max_new_tokens=steps))
+    hf.disable(model)
+    assert torch.isfinite(got).all()
+    err = (got - want).abs().amax(dim=(1, 2))
+    assert float(err.max()) < tol, (int(err.argmax()), float(err.max()))
+    engine = cache.layers[0].engine
+    split = {engine.launch_plan(t, 0.0)[4] > 1 for t in range(9, 9 + steps)}
+    assert split == {False, True}, "the decode never crossed from unsplit to sequence-split launches"
