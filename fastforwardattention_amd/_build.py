@@ -66,9 +66,24 @@ def _run(cmd):
 
 
 def build_lib() -> Path:
-    srcs = [CSRC / "ffa_kernels.hip", CSRC / "ffa_api.cpp", CSRC / "ffa_plan.cpp"]
+    """The device code is four translation units (the decode kernels once per element type, the
+    rest), compiled side by side into objects under build/, then linked with the host sources."""
     hipcc = ROCM / "bin" / "hipcc"
-    _run([hipcc, *HIPCC_FLAGS, f"-I{INCLUDE}", f"-I{CSRC}", *srcs, "-o", LIB_PATH])
+    units = ["ffa_decode_f16.hip", "ffa_decode_bf16.hip", "ffa_decode_f32.hip", "ffa_kernels.hip"]
+    obj_dir = PKG_DIR / "build"
+    obj_dir.mkdir(exist_ok=True)
+    flags = [f for f in HIPCC_FLAGS if f != "-shared"]
+    procs = []
+    for u in units:
+        cmd = [str(hipcc), *flags, "-c", f"-I{INCLUDE}", f"-I{CSRC}", str(CSRC / u), "-o", str(obj_dir / (u + ".o"))]
+        print("+", " ".join(cmd), flush=True)
+        procs.append((u, subprocess.Popen(cmd)))
+    failed = [u for u, p in procs if p.wait() != 0]
+    if failed:
+        raise RuntimeError(f"hipcc failed on {failed}")
+    objs = [obj_dir / (u + ".o") for u in units]
+    _run([hipcc, *HIPCC_FLAGS, f"-I{INCLUDE}", f"-I{CSRC}", *objs, CSRC / "ffa_api.cpp", CSRC / "ffa_plan.cpp",
+          "-o", LIB_PATH])
     LIB_HASH.write_text(lib_source_hash())
     return LIB_PATH
 

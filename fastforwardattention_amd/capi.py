@@ -84,7 +84,7 @@ SIGNATURES = {
     "ffa_attention_ex": (_i, [_i, _i, _i, _i, _i, _f, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _f, _PLAN_P, _i, _TT_P,
                               _BI_P, _vp, _sz, _vp]),
     "ffa_attention_static_scratch": (_i, [_i, _i, _i, _i, _i, _f, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _f,
-                                          _PLAN_P, _i, _vp]),
+                                          _PLAN_P, _i, _TT_P, _BI_P, _vp]),
 }
 
 _lib = None

@@ -36,7 +36,7 @@ int validate_decode(const DecodeArgs& a) {
 
 int run_decode(const DecodeArgs& args, const ffa_launch_plan* user_plan, void* workspace,
                size_t workspace_bytes) {
-    DecodeArgs a = args;
+    const DecodeArgs& a = args;
     int st = validate_decode(a);
     if (st != FFA_OK) return st;
     const int plan_prec = planner_precision(a.precision);
@@ -51,50 +51,54 @@ int run_decode(const DecodeArgs& args, const ffa_launch_plan* user_plan, void* w
         st = plan_launch(plan_prec, a.B, a.H, a.Dh, a.t, a.p, /*use_default=*/0, cus, &plan);
         if (st == FFA_OK && diag && plan.kind == FFA_LAUNCH_SPLIT)
             st = plan_launch(plan_prec, a.B, a.H, a.Dh, a.t, 1.f, 0, cus, &plan);
-        // The kernels with several lanes per key read a sample's own caches only.
-        if (st == FFA_OK && a.cache_indir != nullptr && plan.threads_per_key > 1)
-            st = plan_launch_ex(plan_prec, a.B, a.H, a.Dh, a.t, a.p, 0, cus, /*use_table=*/0, &plan);
         if (st != FFA_OK) return st;
     }
     st = validate_plan(plan, plan_prec, a.Dh, a.B * a.H, a.t, a.p);
     if (st != FFA_OK) return st;
     if (diag && plan.kind == FFA_LAUNCH_SPLIT) return FFA_ERR_PLAN;
-    if (a.cache_indir != nullptr && plan.threads_per_key > 1) return FFA_ERR_PLAN;
 
-    // Workspace layout: [arrival counters][transformed token (only with a transform)][what the
-    // plan needs].  The counters are the only words that persist from call to call, so nothing
-    // else may ever be placed on them, whatever the plan of this step or of an earlier one is.
+    // Workspace layout: [arrival counters][what the plan needs].  The counters are the only
+    // words that persist from call to call; nothing else is ever placed on them.
     WorkspaceView ws = {nullptr, nullptr, nullptr, nullptr, 0};
     const int bh = a.B * a.H;
     const int split_heads = bh - plan.whole_heads;
-    const size_t need = decode_workspace_bytes(plan, bh, a.Dh, a.Lmax, a.transforms_token());
+    const size_t need = plan_workspace_bytes(plan, bh, a.Dh, a.Lmax);
     if (need > 0) {
         if (workspace == nullptr || workspace_bytes < need) return FFA_ERR_WORKSPACE;
         if (!aligned16(workspace)) return FFA_ERR_ALIGNMENT;
-    }
-    char* base = static_cast<char*>(workspace);
-    if (need > 0) {
+        char* base = static_cast<char*>(workspace);
         ws.cnt = reinterpret_cast<unsigned int*>(base);
         base += workspace_counter_bytes(bh);
-    }
-    if (a.transforms_token()) {
-        a.token_scratch = base;
-        base += token_scratch_bytes(bh, a.Dh);
-    }
-    if (plan.kind == FFA_LAUNCH_TWO_PASS) {
-        // [piece (max, sum)][partial outputs][scores]
-        ws.ml = reinterpret_cast<float*>(base);
-        base += align_up((size_t)bh * plan.n_splits * 2 * sizeof(float), 256);
-        ws.acc = reinterpret_cast<float*>(base);
-        base += align_up((size_t)bh * plan.n_splits * a.Dh * sizeof(float), 256);
-        ws.scores = reinterpret_cast<float*>(base);
-        ws.score_stride = score_stride_for(a.Lmax);
-    } else if (plan.kind == FFA_LAUNCH_SPLIT && plan.n_splits > 1 && split_heads > 0) {
-        ws.ml = reinterpret_cast<float*>(base);
-        ws.acc = reinterpret_cast<float*>(
-            base + align_up((size_t)split_heads * plan.n_splits * 2 * sizeof(float), 256));
+        if (plan.kind == FFA_LAUNCH_TWO_PASS) {
+            // [piece (max, sum)][partial outputs][scores]
+            ws.ml = reinterpret_cast<float*>(base);
+            base += align_up((size_t)bh * plan.n_splits * 2 * sizeof(float), 256);
+            ws.acc = reinterpret_cast<float*>(base);
+            base += align_up((size_t)bh * plan.n_splits * a.Dh * sizeof(float), 256);
+            ws.scores = reinterpret_cast<float*>(base);
+            ws.score_stride = score_stride_for(a.Lmax);
+        } else {
+            ws.ml = reinterpret_cast<float*>(base);
+            ws.acc = reinterpret_cast<float*>(
+                base + align_up((size_t)split_heads * plan.n_splits * 2 * sizeof(float), 256));
+        }
     }
     return launch_decode(a, plan, ws);
+}
+
+// Optional parts of a decode call: token transform and beam indirection.
+int apply_options(DecodeArgs& a, const ffa_token_transform* transform, const ffa_beam_indirection* beams) {
+    if (transform != nullptr) {
+        a.q_bias = transform->q_bias; a.k_bias = transform->k_bias; a.v_bias = transform->v_bias;
+        a.rotary_dim = transform->rotary_embedding_dim;
+        a.rotary_base = transform->rotary_base > 0.f ? transform->rotary_base : 10000.f;
+    }
+    if (beams != nullptr) {
+        if (beams->cache_indir == nullptr) return FFA_ERR_BEAM;
+        a.cache_indir = beams->cache_indir;
+        a.beam_width = beams->beam_width;
+    }
+    return FFA_OK;
 }
 
 int run_init_cache(int precision, void* k_dst, void* v_dst, const void* k_src, const void* v_src,
@@ -169,7 +173,7 @@ size_t ffa_workspace_bytes(int batch_size, int head_num, int head_dim, int max_s
     const int n_splits = max_splits_for(bh, max_seq_len);
     const size_t exact = workspace_bytes_for(bh, bh, head_dim, n_splits);
     const size_t two_pass = two_pass_workspace_bytes(bh, head_dim, n_splits, max_seq_len);
-    return align_up(exact > two_pass ? exact : two_pass, 256) + token_scratch_bytes(bh, head_dim);
+    return align_up(exact > two_pass ? exact : two_pass, 256);
 }
 
 int ffa_workspace_init(void* workspace, size_t workspace_bytes, void* stream) {
@@ -232,16 +236,8 @@ int ffa_attention_ex(int precision, int batch_size, int head_num, int head_dim, 
     a.right_or_no_padding = right_or_no_padding;
     a.kept_count = nullptr; a.skip_mask = nullptr;
     a.stream = stream;
-    if (transform != nullptr) {
-        a.q_bias = transform->q_bias; a.k_bias = transform->k_bias; a.v_bias = transform->v_bias;
-        a.rotary_dim = transform->rotary_embedding_dim;
-        a.rotary_base = transform->rotary_base > 0.f ? transform->rotary_base : 10000.f;
-    }
-    if (beams != nullptr) {
-        if (beams->cache_indir == nullptr) return FFA_ERR_BEAM;
-        a.cache_indir = beams->cache_indir;
-        a.beam_width = beams->beam_width;
-    }
+    const int st = apply_options(a, transform, beams);
+    if (st != FFA_OK) return st;
     return run_decode(a, plan, workspace, workspace_bytes);
 }
 
@@ -249,7 +245,9 @@ int ffa_attention_static_scratch(int precision, int batch_size, int head_num, in
                                   int max_seq_len, float softmax_scale, int t, const void* q,
                                   const void* k, const void* v, void* k_cache, void* v_cache,
                                   void* out, const int* seq_lengths, float prob_thresh,
-                                  const ffa_launch_plan* plan, int right_or_no_padding, void* stream) {
+                                  const ffa_launch_plan* plan, int right_or_no_padding,
+                                  const ffa_token_transform* transform,
+                                  const ffa_beam_indirection* beams, void* stream) {
     DecodeArgs a;
     a.precision = precision;
     a.B = batch_size; a.H = head_num; a.Dh = head_dim; a.Lmax = max_seq_len; a.t = t;
@@ -260,7 +258,9 @@ int ffa_attention_static_scratch(int precision, int batch_size, int head_num, in
     a.right_or_no_padding = right_or_no_padding;
     a.kept_count = nullptr; a.skip_mask = nullptr;
     a.stream = stream;
-    int st = validate_decode(a);
+    int st = apply_options(a, transform, beams);
+    if (st != FFA_OK) return st;
+    st = validate_decode(a);
     if (st != FFA_OK) return st;
     ffa_launch_plan chosen;
     if (plan != nullptr) {

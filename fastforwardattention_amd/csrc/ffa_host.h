@@ -38,7 +38,6 @@ struct DecodeArgs {
     const void *q_bias = nullptr, *k_bias = nullptr, *v_bias = nullptr;  // [H, Dh]
     int rotary_dim = 0;
     float rotary_base = 10000.f;
-    void* token_scratch = nullptr;  // 3 * B*H*Dh elements: the transformed q, k, v
     // Beam-search indirection (optional): source beam of every cached key, [B, Lmax].
     const int* cache_indir = nullptr;
     int beam_width = 1;
@@ -46,6 +45,40 @@ struct DecodeArgs {
     bool transforms_token() const { return q_bias || k_bias || v_bias || rotary_dim > 0; }
 };
 
+
+// Kernel parameters of one decode launch (passed by value).
+struct DecodeParams {
+    const void* q;
+    const void* k;
+    const void* v;
+    void* k_cache;
+    void* v_cache;
+    void* out;
+    const int* seq_lengths;
+    float* ws_acc;         // [BH, n_splits, Dh]
+    float* ws_ml;          // [BH, n_splits, 2]
+    unsigned int* ws_cnt;  // [BH]
+    float* ws_scores;      // [BH, score_stride] raw q.k of the two-pass path
+    int score_stride;      // floats per (b,h) row of ws_scores, a multiple of 64
+    unsigned int* kept_count;
+    unsigned char* skip_mask;
+    int B, H, Lmax, t;
+    float scale_log2e;  // softmax_scale * log2(e): scores live in the exp2 domain
+    float p;
+    int right_or_no_padding;
+    int n_splits, tiles_per_split;
+    unsigned split_magic;  // floor(2^32 / n_splits) + 1, or 0 for n_splits = 1: quotients without a division
+    int n_whole;  // (b,h) pairs [0, n_whole) get one workgroup each; the rest are split
+    int bh_total;
+    int combine;  // FFA_COMBINE_*
+    const int* cache_indir;  // [B, Lmax] source beam of every cached key, or nullptr
+    int beam_width;          // samples per beam group (>= 1)
+    // Transform of the new token (all optional): biases [H, Dh], rotary embedding of q and k.
+    const void *q_bias, *k_bias, *v_bias;
+    int rotary_dim;          // 0 = none
+    int xform;               // any bias or a rotary embedding present
+    double rotary_coef;      // -2 log2(base) / rotary_dim: angle of pair z = pos * 2^(z * coef)
+};
 
 // Carved-up workspace for a given plan.
 struct WorkspaceView {
@@ -59,10 +92,6 @@ struct WorkspaceView {
 inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 
 inline int num_tiles(int t) { return t / kTileKeys + 1; }  // keys 0..t inclusive
-
-// Scratch for the transformed new token (q, k, v), sized for the widest element; it sits behind
-// whatever the launch plan itself needs of the workspace.
-inline size_t token_scratch_bytes(int bh, int head_dim) { return align_up((size_t)3 * bh * head_dim * 4, 256); }
 
 // Dynamic LDS of the one-workgroup-per-(b,h) kernel: the larger of the score buffer and
 // the cross-wave merge buffer.
@@ -109,15 +138,6 @@ inline size_t plan_workspace_bytes(const ffa_launch_plan& plan, int bh, int head
     return 0;
 }
 
-// Bytes of workspace one decode call touches: the counter block always leads, the transformed
-// token (if any) follows it, the plan's own regions come last.
-inline size_t decode_workspace_bytes(const ffa_launch_plan& plan, int bh, int head_dim, int max_seq_len,
-                                     bool transforms_token) {
-    const size_t plan_bytes = plan_workspace_bytes(plan, bh, head_dim, max_seq_len);
-    if (!transforms_token) return plan_bytes;
-    return (plan_bytes > 0 ? plan_bytes : workspace_counter_bytes(bh)) + token_scratch_bytes(bh, head_dim);
-}
-
 // Size of the library's own scratch array (one per GPU, held until the process ends), used by
 // ffa_attention_static_scratch in place of a caller-owned workspace.
 constexpr size_t kStaticScratchBytes = FFA_STATIC_SCRATCH_BYTES;
@@ -131,8 +151,14 @@ int plan_launch_ex(int precision, int B, int H, int Dh, int t, float p, int use_
 int validate_plan(const ffa_launch_plan& plan, int precision, int head_dim, int bh, int t, float p);
 bool tpk_supported(int precision, int head_dim, int tpk);
 
-// launchers (ffa_kernels.hip)
+// launchers (ffa_kernels.hip; the decode kernels of each element type are a translation unit of
+// their own: ffa_decode_f16.hip, ffa_decode_bf16.hip, ffa_decode_f32.hip)
 int launch_decode(const DecodeArgs& a, const ffa_launch_plan& plan, const WorkspaceView& ws);
+int launch_decode_f16(const DecodeParams& P, int head_dim, const ffa_launch_plan& plan, void* stream);
+int launch_decode_bf16(const DecodeParams& P, int head_dim, const ffa_launch_plan& plan, void* stream);
+int launch_decode_f32(const DecodeParams& P, int head_dim, const ffa_launch_plan& plan, void* stream);
+constexpr int kMaxDevices = 64;
+int current_device();  // index of the current HIP device, -1 if none or beyond kMaxDevices
 int launch_init_cache(int precision, void* k_dst, void* v_dst, const void* k_src,
                       const void* v_src, int B, int H, int L, int Lmax, int Dh, void* stream);
 int launch_fill_u32(unsigned int* p, size_t n, unsigned int v, void* stream);

@@ -208,7 +208,9 @@ bool tpk_supported(int precision, int head_dim, int tpk) {
 
 int validate_plan(const ffa_launch_plan& plan, int precision, int head_dim, int bh, int t, float p) {
     const int w = plan.waves_per_wg;
-    if (w != 1 && w != 2 && w != 4 && w != 8 && w != 16) return FFA_ERR_PLAN;
+    // Powers of two up to 16; the exact split kernel (one lane per key) also takes 3, 5, 6, 7.
+    const bool pow2 = w == 1 || w == 2 || w == 4 || w == 8 || w == 16;
+    if (!pow2 && !(plan.kind == FFA_LAUNCH_SPLIT && plan.threads_per_key == 1 && w >= 1 && w <= 8)) return FFA_ERR_PLAN;
     const int tpk = plan.threads_per_key;
     if ((tpk != 1 && tpk != 2 && tpk != 4) || plan.keys_per_wave != kTileKeys / tpk) return FFA_ERR_PLAN;
     // More than one lane per key exists in the exact split kernel only, with 4 or 8 waves.

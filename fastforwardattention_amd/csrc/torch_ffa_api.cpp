@@ -252,11 +252,8 @@ private:
         ffa_launch_plan plan;
         const bool diag = kept != nullptr || mask != nullptr;
         // The default launch keeps diagnostics at any length; the exact split kernel has none.
-        // Plans with several lanes per key (only the measured table holds such) take no beam
-        // indirection: with one, plan by the rules alone.
-        check_status((beams != nullptr ? ffa_plan_launch_rules : ffa_plan_launch)(
-                         plan_precision(precision), d.B, d.H, d.Dh, t, prob_thresh,
-                         (ft_kernel_launch || diag) ? 1 : 0, 0, &plan),
+        check_status(ffa_plan_launch(plan_precision(precision), d.B, d.H, d.Dh, t, prob_thresh,
+                                     (ft_kernel_launch || diag) ? 1 : 0, 0, &plan),
                      "launch planning");
         if (transform != nullptr || beams != nullptr) {
             TORCH_CHECK(!diag, "ff_attention: diagnostics cannot be combined with a token transform or beams");

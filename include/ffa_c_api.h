@@ -81,7 +81,8 @@ typedef enum ffa_status {
 /* Replaces the (tpb, tpv, tpk) triple of kernel_launch_utils.h:135-180. */
 typedef struct ffa_launch_plan {
     int32_t kind;             /* FFA_LAUNCH_*                                              */
-    int32_t waves_per_wg;     /* wave64 wavefronts per workgroup: 1, 2, 4, 8 or 16         */
+    int32_t waves_per_wg;     /* wave64 wavefronts per workgroup: 1, 2, 4, 8 or 16; also   */
+                              /* 3, 5, 6, 7 in FFA_LAUNCH_SPLIT plans with one lane per key */
     int32_t threads_per_key;  /* lanes cooperating on one key's q.k: 1, or 2 / 4 in        */
                               /* FFA_LAUNCH_SPLIT plans with 4 or 8 waves (head dims 64,   */
                               /* 128 and, for 4 lanes, 256 in fp16 / 128 in fp32)          */
@@ -124,8 +125,7 @@ int ffa_plan_launch_rules(int precision, int batch_size, int head_num, int head_
                           int compute_units, ffa_launch_plan* plan);
 
 /* Bytes of device workspace sufficient for ANY plan this library produces for the
- * given problem (arrival counters, split partials, two-pass scores, the transformed token
- * of ffa_attention_ex). */
+ * given problem (arrival counters, split partials, two-pass scores). */
 size_t ffa_workspace_bytes(int batch_size, int head_num, int head_dim, int max_seq_len);
 
 /* Zero a workspace (what matters are the arrival counters at its head; the buffer may be of
@@ -223,9 +223,8 @@ int ffa_attention_diag(int precision, int batch_size, int head_num, int head_dim
  *              beams of a group must be at the same length (same t, same seq_lengths entry):
  *              a beam's slot t is written in the launch in which its siblings read the slots
  *              below theirs.  batch_size must be a multiple of beam_width and
- *              beam_width * head_num * max_seq_len must stay below 2^31 (FFA_ERR_BEAM);
- *              launch plans with more than one lane per key do not take an indirection
- *              (FFA_ERR_PLAN; a NULL plan never picks one).
+ *              beam_width * head_num * max_seq_len must stay below 2^31 (FFA_ERR_BEAM).
+ *              Every launch plan takes an indirection.
  */
 typedef struct ffa_token_transform {
     const void* q_bias;
@@ -260,7 +259,7 @@ int ffa_attention_ex(int precision, int batch_size, int head_num, int head_dim, 
  *     streams, two host threads) race; calls on one stream are ordered and safe;
  *   - the arrival counters of the call's (batch, head) pairs are cleared by a small kernel
  *     on `stream` ahead of the decode kernel.
- * Arguments as ffa_attention_diag, without workspace and diagnostics.
+ * Arguments as ffa_attention_ex (transform and beams may be NULL), without the workspace.
  */
 #define FFA_STATIC_SCRATCH_BYTES (4u << 20)
 int ffa_attention_static_scratch(int precision, int batch_size, int head_num, int head_dim,
@@ -268,7 +267,8 @@ int ffa_attention_static_scratch(int precision, int batch_size, int head_num, in
                                   const void* k, const void* v, void* k_cache, void* v_cache,
                                   void* out, const int* seq_lengths, float prob_thresh,
                                   const ffa_launch_plan* plan, int right_or_no_padding,
-                                  void* stream);
+                                  const ffa_token_transform* transform,
+                                  const ffa_beam_indirection* beams, void* stream);
 
 #ifdef __cplusplus
 }

@@ -108,8 +108,8 @@ def test_pruned_diag_and_stream():
     assert torch.equal(kept.long(), L - mask[:, :, :L].sum(-1).long())
     assert 0 < mask.float().mean() < 1
     assert float((out.float() - exact.float()).abs().max()) < 0.2
-    plain = ffa.attention(q, k, v, 0.5, L, 5e-2)
-    assert torch.equal(plain, out)
+    plain = ffa.attention(q, k, v, 0.5, L, 5e-2)     # another launch plan: the same rule, another order of summation
+    assert float((plain.float() - out.float()).abs().max()) <= 1e-3
     # a side stream: the extension launches on torch's current stream
     s = torch.cuda.Stream()
     s.wait_stream(torch.cuda.current_stream())

@@ -40,6 +40,10 @@ def _plans(prec, B, H, Dh, t):
             plans.append((f"split_w{waves}_tps{tps}", capi.make_plan(capi.FFA_LAUNCH_SPLIT, waves, ns, tps)))
             plans.append((f"split_w{waves}_tps{tps}_mergekernel",
                           capi.make_plan(capi.FFA_LAUNCH_SPLIT, waves, ns, tps, capi.FFA_COMBINE_KERNEL)))
+    for waves, tps in [(3, 2), (5, 3), (6, 1), (7, ntiles)]:       # workgroups of 3, 5, 6, 7 waves
+        ns = -(-ntiles // tps)
+        if ns <= 128:
+            plans.append((f"split_w{waves}_tps{tps}", capi.make_plan(capi.FFA_LAUNCH_SPLIT, waves, ns, tps)))
     # 2 and 4 lanes per key (tiles of 32 and 16 keys), where the kernel exists for this shape
     nch = Dh * (prec // 8) // 16
     for tpk in (2, 4):

@@ -30,7 +30,7 @@ def _both(sess, q, k, v, scale, t, p, plan):
         if static:
             rc = sess.lib.ffa_attention_static_scratch(
                 sess.precision, sess.B, sess.H, sess.Dh, sess.Lmax, float(scale), int(t), ptr(qd), ptr(kd), ptr(vd),
-                ptr(sess.k_cache), ptr(sess.v_cache), ptr(out), None, float(p), plan_p, 1, None)
+                ptr(sess.k_cache), ptr(sess.v_cache), ptr(out), None, float(p), plan_p, 1, None, None, None)
         else:
             rc = sess.lib.ffa_attention_diag(
                 sess.precision, sess.B, sess.H, sess.Dh, sess.Lmax, float(scale), int(t), ptr(qd), ptr(kd), ptr(vd),
@@ -81,7 +81,7 @@ def test_static_scratch_rejects_oversized_plan():
     nt = t // 64 + 1
     plan = capi.make_plan(capi.FFA_LAUNCH_TWO_PASS, 4, 4, -(-nt // 4))
     rc = sess.lib.ffa_attention_static_scratch(16, B, H, Dh, t + 1, 0.125, t, ptr(x), ptr(x), ptr(x), ptr(sess.k_cache),
-                                                ptr(sess.v_cache), ptr(out), None, 0.01, C.byref(plan), 1, None)
+                                                ptr(sess.v_cache), ptr(out), None, 0.01, C.byref(plan), 1, None, None, None)
     assert rc == capi.FFA_ERR_SCRATCH_LIMIT
     assert b"scratch" in sess.lib.ffa_status_string(rc)
     torch.cuda.synchronize()
@@ -102,7 +102,7 @@ def test_static_scratch_in_a_captured_graph():
     def call(stream_ptr):
         rc = sess.lib.ffa_attention_static_scratch(16, B, H, Dh, t + 2, 0.125, t, ptr(qd), ptr(kd), ptr(vd),
                                                     ptr(sess.k_cache), ptr(sess.v_cache), ptr(out), None, 0.0, None, 1,
-                                                    stream_ptr)
+                                                    None, None, stream_ptr)
         assert rc == capi.FFA_OK
     call(None)
     torch.cuda.synchronize()
