@@ -265,6 +265,18 @@ __device__ __forceinline__ bool setup_q(const DecodeParams& P, int bh, int h, in
     }
 }
 
+// The transform of q alone, by a tile wave, from raw pairs it loaded before its first tile: the
+// arithmetic runs while that tile is on its way.
+template <typename T, int DH>
+__device__ __forceinline__ void transform_q_only(const DecodeParams& P, const RawToken<T, DH>& raw, int tlen, int first,
+                                                 TokenLds<T, DH>& s, int lane) {
+    transform_token<T, DH>(P, raw, max(tlen - first, 0), /*with_kv=*/false, reinterpret_cast<T*>(s.q),
+                           reinterpret_cast<T*>(s.k), reinterpret_cast<T*>(s.v), lane);
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
 // The new token in the token wave's registers: lane c < NCH holds 16-byte chunk c of q, k, v
 // (after the transform, if any).
 struct TokenRegs {
@@ -732,7 +744,6 @@ __global__ void __launch_bounds__((NW + 1) * 64) ffa_decode_split_kernel(const D
         if (has_token) tok = token_wave_state<T, DH>(P, bh, bh - b * P.H, tlen, first, s_tok, m_run, l_run, acc, lane);
     } else {
     uint4 q_reg[G::QREG];
-    const bool q_in_lds = setup_q<T, DH>(P, bh, bh - b * P.H, tlen, first, /*token_wave=*/false, s_tok, q_reg, lane);
 
     // Scores, online softmax and P.V of one tile whose first load groups are in kv / vv.
     // QL: q is read from LDS (wide heads, transformed token) instead of SGPRs.
@@ -788,9 +799,9 @@ __global__ void __launch_bounds__((NW + 1) * 64) ffa_decode_split_kernel(const D
     const TileOrder order(tile_lo, tile_hi, (unsigned)(bh * n_splits + split));
     // One loop per source of q, each with a straight-line body (a branch on the source inside
     // the loop lets the compiler hoist code of the tile's arithmetic in between its loads).
-    auto walk_tiles = [&](auto ql) {
-        int src_next = wave < order.n ? beams.beam(min(order.at(wave) * kWave + lane, last_key), tlen) : 0;
-        for (int idx = wave; idx < order.n; idx += NW) {
+    auto walk_tiles = [&](auto ql, int from) {
+        int src_next = from < order.n ? beams.beam(min(order.at(from) * kWave + lane, last_key), tlen) : 0;
+        for (int idx = from; idx < order.n; idx += NW) {
             const int tile = order.at(idx);
             const int src = src_next;
             if constexpr (BEAM)
@@ -801,11 +812,28 @@ __global__ void __launch_bounds__((NW + 1) * 64) ffa_decode_split_kernel(const D
             compute_tile(ql, kv, vv, tile, src);
         }
     };
-    if constexpr (G::Q_LDS) {
-        walk_tiles(std::true_type{});
+    if (P.xform) {
+        // With a transform: raw pairs of q first (small loads at the head of the queue), then the
+        // loads of the wave's first tile, then the fp64 arithmetic in the shadow of that tile.
+        if (wave < order.n) {
+            const RawToken<T, DH> raw = token_raw_load<T, DH>(P, bh, bh - b * P.H, /*with_kv=*/false, lane);
+            const int tile = order.at(wave);
+            const int src = beams.beam(min(tile * kWave + lane, last_key), tlen);
+            uint4 kv[CG], vv[VG];
+            load_tile(kv, vv, tile, src);
+            __builtin_amdgcn_sched_barrier(0);
+            transform_q_only<T, DH>(P, raw, tlen, first, s_tok, lane);
+            compute_tile(std::true_type{}, kv, vv, tile, src);
+            walk_tiles(std::true_type{}, wave + NW);
+        }
     } else {
-        if (q_in_lds) walk_tiles(std::true_type{});
-        else walk_tiles(std::false_type{});
+        const bool q_in_lds = setup_q<T, DH>(P, bh, 0, tlen, first, /*token_wave=*/false, s_tok, q_reg, lane);
+        if constexpr (G::Q_LDS) {
+            (void)q_in_lds;
+            walk_tiles(std::true_type{}, wave);
+        } else {
+            walk_tiles(std::false_type{}, wave);
+        }
     }
     }  // tile waves
 
@@ -889,31 +917,9 @@ __global__ void __launch_bounds__((NW + 1) * 64) ffa_decode_split_tpk_kernel(con
     if (token_wave) {
         if (has_token) tok = token_wave_state<T, DH>(P, bh, bh - b * P.H, tlen, first, s_tok, m_run, l_run, acc, lane);
     } else {
-    // q: this lane's share of the chunks, from memory or, after a transform, from LDS.
-    uint4 q_full[G::QREG];
-    const bool q_in_lds = setup_q<T, DH>(P, bh, bh - b * P.H, tlen, first, /*token_wave=*/false, s_tok, q_full, lane);
-    uint4 q_reg[NK];
-    if (q_in_lds) {
-#pragma unroll
-        for (int i = 0; i < NK; ++i) q_reg[i] = s_tok.q[part * NK + i];
-    } else {
-        const char* qg = reinterpret_cast<const char*>(P.q) + (size_t)bh * DH * sizeof(T);
-#pragma unroll
-        for (int i = 0; i < NK; ++i) q_reg[i] = *reinterpret_cast<const uint4*>(qg + (part * NK + i) * 16);
-    }
-
-    const TileOrder order(tile_lo, tile_hi, (unsigned)(bh * n_splits + split));
-    int src_next = wave < order.n ? beams.beam(min(order.at(wave) * KPT + kl, last_key), tlen) : 0;
-    for (int idx = wave; idx < order.n; idx += NW) {
-        const int tile = order.at(idx);
-        const int src = src_next;
-        if constexpr (BEAM)
-            src_next = idx + NW < order.n ? beams.beam(min(order.at(idx + NW) * KPT + kl, last_key), tlen) : 0;
+    uint4 q_reg[NK];  // this lane's share of q: chunks [part*NK, part*NK + NK)
+    auto compute_tile = [&](uint4 (&kv)[NK], uint4 (&vv)[NV], int tile) {
         const int key = tile * KPT + kl;
-        uint4 kv[NK], vv[NV];
-        load_tile(kv, vv, tile, src);
-        __builtin_amdgcn_sched_barrier(0);
-
         float s = 0.f;
 #pragma unroll
         for (int i = 0; i < NK; ++i) s = dot_chunk(kv[i], q_reg[i], s, T{});
@@ -936,6 +942,48 @@ __global__ void __launch_bounds__((NW + 1) * 64) ffa_decode_split_tpk_kernel(con
 #pragma unroll
         for (int j = 0; j < NV; ++j) fma_chunk(acc, pst[j], vv[j], T{});
         __builtin_amdgcn_wave_barrier();
+    };
+    const TileOrder order(tile_lo, tile_hi, (unsigned)(bh * n_splits + split));
+    auto walk_tiles = [&](int from) {
+        int src_next = from < order.n ? beams.beam(min(order.at(from) * KPT + kl, last_key), tlen) : 0;
+        for (int idx = from; idx < order.n; idx += NW) {
+            const int tile = order.at(idx);
+            const int src = src_next;
+            if constexpr (BEAM)
+                src_next = idx + NW < order.n ? beams.beam(min(order.at(idx + NW) * KPT + kl, last_key), tlen) : 0;
+            uint4 kv[NK], vv[NV];
+            load_tile(kv, vv, tile, src);
+            __builtin_amdgcn_sched_barrier(0);
+            compute_tile(kv, vv, tile);
+        }
+    };
+    if (P.xform) {
+        // As in ffa_decode_split_kernel: raw pairs, first tile's loads, arithmetic in their shadow.
+        if (wave < order.n) {
+            const RawToken<T, DH> raw = token_raw_load<T, DH>(P, bh, bh - b * P.H, /*with_kv=*/false, lane);
+            const int tile = order.at(wave);
+            const int src = beams.beam(min(tile * KPT + kl, last_key), tlen);
+            uint4 kv[NK], vv[NV];
+            load_tile(kv, vv, tile, src);
+            __builtin_amdgcn_sched_barrier(0);
+            transform_q_only<T, DH>(P, raw, tlen, first, s_tok, lane);
+#pragma unroll
+            for (int i = 0; i < NK; ++i) q_reg[i] = s_tok.q[part * NK + i];
+            compute_tile(kv, vv, tile);
+            walk_tiles(wave + NW);
+        }
+    } else {
+        uint4 q_full[G::QREG];
+        const bool q_in_lds = setup_q<T, DH>(P, bh, 0, tlen, first, /*token_wave=*/false, s_tok, q_full, lane);
+        if (q_in_lds) {
+#pragma unroll
+            for (int i = 0; i < NK; ++i) q_reg[i] = s_tok.q[part * NK + i];
+        } else {
+            const char* qg = reinterpret_cast<const char*>(P.q) + (size_t)bh * DH * sizeof(T);
+#pragma unroll
+            for (int i = 0; i < NK; ++i) q_reg[i] = *reinterpret_cast<const uint4*>(qg + (part * NK + i) * 16);
+        }
+        walk_tiles(wave);
     }
     }  // tile waves
     finish_piece<T, DH, NW + 1>(P, bh, split, n_splits, acc, m_run, l_run, s_merge);
