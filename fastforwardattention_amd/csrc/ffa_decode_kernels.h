@@ -750,15 +750,28 @@ __global__ void __launch_bounds__((NW + 1) * 64) ffa_decode_split_kernel(const D
     auto compute_tile = [&](auto ql, uint4 (&kv)[CG], uint4 (&vv)[VG], int tile, int src) {
         constexpr bool QL = decltype(ql)::value;
         const int key = tile * kWave + lane;
-        float s = dot_k_group<T, CG, QL>(kv, 0, q_reg, s_tok.q, 0.f);
+        float s = 0.f;
         if constexpr (NCH > CG) {
+            // Rolling groups: as soon as chunk c of a group has been consumed its registers take
+            // chunk c of the next group, so a wave has a tile's first CG + VG loads in flight and
+            // then tops up one by one.  (Left to itself the compiler hoists a whole second group
+            // of K loads above the first dot product: 24 loads in flight per wave cost 5 % at
+            // 320 pairs x 1000 keys of fp32.)
             const char* kp = beams.k_of(src) + (size_t)min(key, last_key) * 16;
-#pragma unroll 2
-            for (int g = 1; g < NCH / CG; ++g) {
-                uint4 kn[CG];
-                load_k_group<CG>(kn, kp, kstr, g);
-                s = dot_k_group<T, CG, QL>(kn, g, q_reg, s_tok.q, s);
+#pragma unroll
+            for (int g = 0; g < NCH / CG; ++g) {
+#pragma unroll
+                for (int c = 0; c < CG; ++c) {
+                    uint4 qc;
+                    if constexpr (QL) qc = s_tok.q[g * CG + c];
+                    else qc = q_reg[g * CG + c];
+                    s = dot_chunk(kv[c], qc, s, T{});
+                    if (g + 1 < NCH / CG) kv[c] = ld16(kp + (size_t)((g + 1) * CG + c) * kstr);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
             }
+        } else {
+            s = dot_k_group<T, CG, QL>(kv, 0, q_reg, s_tok.q, 0.f);
         }
 
         const bool valid = key < tlen && key >= first;
