@@ -31,6 +31,9 @@ HIP_ARCH = "gfx950"
 HIPCC_FLAGS = [
     f"--offload-arch={HIP_ARCH}", "-O3", "-std=c++17", "-fPIC", "-shared",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    # Leading scalar kernel arguments arrive in SGPRs with the wave (the split kernels take what
+    # their first loads need that way); kernels whose only argument is a struct are unaffected.
+    "-mllvm", "-amdgpu-kernarg-preload-count=14",
     "-Wall", "-Wno-unused-function",
 ]
 
@@ -66,10 +69,12 @@ def _run(cmd):
 
 
 def build_lib() -> Path:
-    """The device code is four translation units (the decode kernels once per element type, the
-    rest), compiled side by side into objects under build/, then linked with the host sources."""
+    """The device code is seven translation units (the decode kernels once per element type and
+    transform switch, the rest), compiled side by side into objects under build/, then linked
+    with the host sources."""
     hipcc = ROCM / "bin" / "hipcc"
-    units = ["ffa_decode_f16.hip", "ffa_decode_bf16.hip", "ffa_decode_f32.hip", "ffa_kernels.hip"]
+    units = ["ffa_decode_f16.hip", "ffa_decode_bf16.hip", "ffa_decode_f32.hip", "ffa_decode_f16_xform.hip",
+             "ffa_decode_bf16_xform.hip", "ffa_decode_f32_xform.hip", "ffa_kernels.hip"]
     obj_dir = PKG_DIR / "build"
     obj_dir.mkdir(exist_ok=True)
     flags = [f for f in HIPCC_FLAGS if f != "-shared"]

@@ -1,0 +1,11 @@
+// Decode kernels of the engine instantiated for one element type (bf16_t), with the bias / rotary transform of the new token:
+// one translation unit per element type and transform switch, so that the six compile in parallel.
+#include "ffa_decode_kernels.h"
+
+namespace ffa {
+
+int launch_decode_bf16_xform(const DecodeParams& P, int head_dim, const ffa_launch_plan& plan, void* stream) {
+    return dispatch_head_dim<bf16_t, true>(P, head_dim, plan, reinterpret_cast<hipStream_t>(stream));
+}
+
+}  // namespace ffa

@@ -45,6 +45,26 @@
 
 namespace ffa {
 
+// What a workgroup needs before it can issue its first cache load travels as leading scalar
+// kernel arguments, which the hardware can place in registers while it launches the wave
+// (kernel-argument preloading); everything else is fetched from the argument block in memory.
+#define HOT_PARAMS_DECL                                                                                      \
+    void *hot_k_cache, void *hot_v_cache, const int *hot_seq_lengths, int hot_Lmax, int hot_t, int hot_n_whole, \
+        int hot_n_splits, unsigned hot_split_magic, int hot_tiles_per_split, const void *hot_q
+#define HOT_PARAMS_USE                                                                                            \
+    hot_k_cache, hot_v_cache, hot_seq_lengths, hot_Lmax, hot_t, hot_n_whole, hot_n_splits, hot_split_magic, \
+        hot_tiles_per_split, hot_q
+#define HOT_PARAMS_OF(P)                                                                                  \
+    (P).k_cache, (P).v_cache, (P).seq_lengths, (P).Lmax, (P).t, (P).n_whole, (P).n_splits, (P).split_magic, \
+        (P).tiles_per_split, (P).q
+__device__ __forceinline__ DecodeParams with_hot_params(const DecodeParams& rest, HOT_PARAMS_DECL) {
+    DecodeParams P = rest;
+    P.k_cache = hot_k_cache; P.v_cache = hot_v_cache; P.seq_lengths = hot_seq_lengths;
+    P.Lmax = hot_Lmax; P.t = hot_t; P.n_whole = hot_n_whole; P.n_splits = hot_n_splits;
+    P.split_magic = hot_split_magic; P.tiles_per_split = hot_tiles_per_split; P.q = hot_q;
+    return P;
+}
+
 // Per-(b) bounds, attention.cu:805-817.  tlen = slot of the new token = number of cached
 // keys; first = first unmasked key.  Values are clamped so that a bad seq_lengths entry
 // can never produce an out-of-bounds access.
@@ -64,23 +84,21 @@ __device__ __forceinline__ void step_bounds(const DecodeParams& P, int b, int& t
 // planner admits): an integer division here would sit in front of every workgroup's first load.
 // r / n_splits for r below 2^25 / n_splits (split_magic = 0 stands for n_splits = 1).
 __device__ __forceinline__ unsigned pair_of(const DecodeParams& P, unsigned r) {
-    return P.split_magic == 0u ? r : __umulhi(r, P.split_magic);
+    const unsigned hi = __umulhi(r, P.split_magic);
+    return P.split_magic == 0u ? r : hi;
 }
 
+// Branch-free on purpose: with a branch in front of them the compiler fetches the kernel
+// arguments in two dependent batches, each a miss of the scalar cache right after a launch.
 struct PieceOf {
     int bh, split, n_splits;
     __device__ __forceinline__ PieceOf(const DecodeParams& P, int wg) {
-        if (wg < P.n_whole) {
-            bh = wg;
-            split = 0;
-            n_splits = 1;
-        } else {
-            const unsigned r = (unsigned)(wg - P.n_whole);
-            const unsigned pair = pair_of(P, r);
-            bh = P.n_whole + (int)pair;
-            split = (int)(r - pair * (unsigned)P.n_splits);
-            n_splits = P.n_splits;
-        }
+        const bool whole = wg < P.n_whole;
+        const unsigned r = (unsigned)(wg - P.n_whole);
+        const unsigned pair = pair_of(P, r);
+        bh = whole ? wg : P.n_whole + (int)pair;
+        split = whole ? 0 : (int)(r - pair * (unsigned)P.n_splits);
+        n_splits = whole ? 1 : P.n_splits;
     }
 };
 
@@ -237,12 +255,12 @@ struct alignas(16) TokenLds {
 // it wrote) and, if it is the token wave, k' and v' as well.  The two sources are kept apart all
 // the way into the tile code: a register array fed from two places costs the plain path its
 // wide scalar loads.
-template <typename T, int DH>
+template <typename T, int DH, bool XFORM>
 __device__ __forceinline__ bool setup_q(const DecodeParams& P, int bh, int h, int tlen, int first, bool token_wave,
                                         TokenLds<T, DH>& s, uint4 (&q_reg)[Geo<T, DH>::QREG], int lane) {
     using G = Geo<T, DH>;
     const uint4* qg = reinterpret_cast<const uint4*>(reinterpret_cast<const char*>(P.q) + (size_t)bh * DH * sizeof(T));
-    if (P.xform) {
+    if constexpr (XFORM) {
         const RawToken<T, DH> raw = token_raw_load<T, DH>(P, bh, h, token_wave, lane);
         transform_token<T, DH>(P, raw, max(tlen - first, 0), token_wave, reinterpret_cast<T*>(s.q),
                                reinterpret_cast<T*>(s.k), reinterpret_cast<T*>(s.v), lane);
@@ -282,12 +300,12 @@ __device__ __forceinline__ void transform_q_only(const DecodeParams& P, const Ra
 struct TokenRegs {
     uint4 q, k, v;
 };
-template <typename T, int DH>
+template <typename T, int DH, bool XFORM>
 __device__ __forceinline__ TokenRegs token_load(const DecodeParams& P, int bh, const TokenLds<T, DH>& s, int lane) {
     constexpr int NCH = Geo<T, DH>::NCH;
     const int c = lane < NCH ? lane : 0;
     TokenRegs r;
-    if (P.xform) {  // setup_q of this wave has put them in LDS
+    if constexpr (XFORM) {  // setup_q of this wave has put them in LDS
         r.q = s.q[c];
         r.k = s.k[c];
         r.v = s.v[c];
@@ -509,14 +527,14 @@ __device__ __forceinline__ void queue_drain(float (&acc)[Elem<T>::X], SurvivorQu
 // barrier, when the tile waves have read all they will read: in the middle of the stream every
 // write turns memory channels around under the reads (measured at 320 pairs x 1000 keys: 0.1 us
 // per launch for 640 small stores).
-template <typename T, int DH>
+template <typename T, int DH, bool XFORM>
 __device__ __forceinline__ TokenRegs token_wave_state(const DecodeParams& P, int bh, int h, int tlen, int first,
                                                       TokenLds<T, DH>& s_tok, float& m_run, float& l_run,
                                                       float (&acc)[Elem<T>::X], int lane) {
     constexpr int NCH = Geo<T, DH>::NCH;
     uint4 q_unused[Geo<T, DH>::QREG];
-    if (P.xform) (void)setup_q<T, DH>(P, bh, h, tlen, first, /*token_wave=*/true, s_tok, q_unused, lane);
-    const TokenRegs tok = token_load<T, DH>(P, bh, s_tok, lane);
+    if constexpr (XFORM) (void)setup_q<T, DH, true>(P, bh, h, tlen, first, /*token_wave=*/true, s_tok, q_unused, lane);
+    const TokenRegs tok = token_load<T, DH, XFORM>(P, bh, s_tok, lane);
     const float s = token_score<T, DH>(tok, lane);
     if (tlen >= first) {  // else the whole sample is masked up to and including the new slot
         m_run = s * P.scale_log2e;
@@ -670,8 +688,10 @@ __device__ __forceinline__ void finish_piece(const DecodeParams& P, int bh, int 
 
 // ---------------------------------------------------------------------------------------
 // Sequence-split exact decode (p == 0).
-template <typename T, int DH, int NW, bool BEAM>
-__global__ void __launch_bounds__((NW + 1) * 64) ffa_decode_split_kernel(const DecodeParams P) {
+template <typename T, int DH, int NW, bool BEAM, bool XFORM>
+__global__ void __launch_bounds__((NW + 1) * 64)
+ffa_decode_split_kernel(HOT_PARAMS_DECL, const DecodeParams P_rest) {
+    const DecodeParams P = with_hot_params(P_rest, HOT_PARAMS_USE);
     using G = Geo<T, DH>;
     constexpr int X = G::X, NCH = G::NCH, LPR = G::LPR, RPI = G::RPI, NVL = G::NVL;
     constexpr int VG = G::VG;  // V loads kept in flight per group
@@ -690,7 +710,7 @@ __global__ void __launch_bounds__((NW + 1) * 64) ffa_decode_split_kernel(const D
     // cross-workgroup merges (a chain of memory round trips) finish in their shadow.
     const PieceOf piece(P, (int)blockIdx.x);
     const int bh = piece.bh, split = piece.split, n_splits = piece.n_splits;
-    const bool need_b = P.seq_lengths != nullptr || BEAM || P.xform;
+    const bool need_b = P.seq_lengths != nullptr || BEAM || XFORM;
     const int b = need_b ? bh / P.H : 0;
 
     int tlen, first;
@@ -741,7 +761,7 @@ __global__ void __launch_bounds__((NW + 1) * 64) ffa_decode_split_kernel(const D
     TokenRegs tok;
     const bool has_token = token_wave && split == n_splits - 1;
     if (token_wave) {
-        if (has_token) tok = token_wave_state<T, DH>(P, bh, bh - b * P.H, tlen, first, s_tok, m_run, l_run, acc, lane);
+        if (has_token) tok = token_wave_state<T, DH, XFORM>(P, bh, bh - b * P.H, tlen, first, s_tok, m_run, l_run, acc, lane);
     } else {
     uint4 q_reg[G::QREG];
 
@@ -794,10 +814,16 @@ __global__ void __launch_bounds__((NW + 1) * 64) ffa_decode_split_kernel(const D
 #pragma unroll
         for (int g = 0; g < NVL / VG; ++g) {
             uint4 vn[VG];
-            if (g + 1 < NVL / VG) load_v_group(vn, tile, g + 1, src);
+            if (g + 1 < NVL / VG) {
+                // The next group goes out as a block before this one is consumed (left alone, the
+                // compiler may sink each load next to its use: one round trip per pair of loads).
+                load_v_group(vn, tile, g + 1, src);
+                __builtin_amdgcn_sched_barrier(0);
+            }
 #pragma unroll
             for (int j = 0; j < VG; ++j) fma_chunk(acc, pst[g * VG + j], vv[j], T{});
             if (g + 1 < NVL / VG) {
+                __builtin_amdgcn_sched_barrier(0);  // one group ahead, not more
 #pragma unroll
                 for (int j = 0; j < VG; ++j) vv[j] = vn[j];
             }
@@ -825,7 +851,7 @@ __global__ void __launch_bounds__((NW + 1) * 64) ffa_decode_split_kernel(const D
             compute_tile(ql, kv, vv, tile, src);
         }
     };
-    if (P.xform) {
+    if constexpr (XFORM) {
         // With a transform: raw pairs of q first (small loads at the head of the queue), then the
         // loads of the wave's first tile, then the fp64 arithmetic in the shadow of that tile.
         if (wave < order.n) {
@@ -840,7 +866,7 @@ __global__ void __launch_bounds__((NW + 1) * 64) ffa_decode_split_kernel(const D
             walk_tiles(std::true_type{}, wave + NW);
         }
     } else {
-        const bool q_in_lds = setup_q<T, DH>(P, bh, 0, tlen, first, /*token_wave=*/false, s_tok, q_reg, lane);
+        const bool q_in_lds = setup_q<T, DH, false>(P, bh, 0, tlen, first, /*token_wave=*/false, s_tok, q_reg, lane);
         if constexpr (G::Q_LDS) {
             (void)q_in_lds;
             walk_tiles(std::true_type{}, wave);
@@ -864,8 +890,10 @@ __global__ void __launch_bounds__((NW + 1) * 64) ffa_decode_split_kernel(const D
 // at Dh = 256 a tile whose 16 loads are all in flight at once where one lane per key needs
 // four dependent groups of loads.  Pieces are cut in units of 64 keys exactly as in
 // ffa_decode_split_kernel, with which this kernel shares its epilogue.
-template <typename T, int DH, int NW, int TPK, bool BEAM>
-__global__ void __launch_bounds__((NW + 1) * 64) ffa_decode_split_tpk_kernel(const DecodeParams P) {
+template <typename T, int DH, int NW, int TPK, bool BEAM, bool XFORM>
+__global__ void __launch_bounds__((NW + 1) * 64)
+ffa_decode_split_tpk_kernel(HOT_PARAMS_DECL, const DecodeParams P_rest) {
+    const DecodeParams P = with_hot_params(P_rest, HOT_PARAMS_USE);
     using G = Geo<T, DH>;
     constexpr int X = G::X, NCH = G::NCH, LPR = G::LPR, RPI = G::RPI;
     constexpr int KPT = kWave / TPK;   // keys per tile
@@ -882,7 +910,7 @@ __global__ void __launch_bounds__((NW + 1) * 64) ffa_decode_split_tpk_kernel(con
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const PieceOf piece(P, (int)blockIdx.x);
     const int bh = piece.bh, split = piece.split, n_splits = piece.n_splits;
-    const bool need_b = P.seq_lengths != nullptr || BEAM || P.xform;
+    const bool need_b = P.seq_lengths != nullptr || BEAM || XFORM;
     const int b = need_b ? bh / P.H : 0;
     int tlen, first;
     step_bounds(P, b, tlen, first);
@@ -928,7 +956,7 @@ __global__ void __launch_bounds__((NW + 1) * 64) ffa_decode_split_tpk_kernel(con
     TokenRegs tok;
     const bool has_token = token_wave && split == n_splits - 1;
     if (token_wave) {
-        if (has_token) tok = token_wave_state<T, DH>(P, bh, bh - b * P.H, tlen, first, s_tok, m_run, l_run, acc, lane);
+        if (has_token) tok = token_wave_state<T, DH, XFORM>(P, bh, bh - b * P.H, tlen, first, s_tok, m_run, l_run, acc, lane);
     } else {
     uint4 q_reg[NK];  // this lane's share of q: chunks [part*NK, part*NK + NK)
     auto compute_tile = [&](uint4 (&kv)[NK], uint4 (&vv)[NV], int tile) {
@@ -970,7 +998,7 @@ __global__ void __launch_bounds__((NW + 1) * 64) ffa_decode_split_tpk_kernel(con
             compute_tile(kv, vv, tile);
         }
     };
-    if (P.xform) {
+    if constexpr (XFORM) {
         // As in ffa_decode_split_kernel: raw pairs, first tile's loads, arithmetic in their shadow.
         if (wave < order.n) {
             const RawToken<T, DH> raw = token_raw_load<T, DH>(P, bh, bh - b * P.H, /*with_kv=*/false, lane);
@@ -987,7 +1015,7 @@ __global__ void __launch_bounds__((NW + 1) * 64) ffa_decode_split_tpk_kernel(con
         }
     } else {
         uint4 q_full[G::QREG];
-        const bool q_in_lds = setup_q<T, DH>(P, bh, 0, tlen, first, /*token_wave=*/false, s_tok, q_full, lane);
+        const bool q_in_lds = setup_q<T, DH, false>(P, bh, 0, tlen, first, /*token_wave=*/false, s_tok, q_full, lane);
         if (q_in_lds) {
 #pragma unroll
             for (int i = 0; i < NK; ++i) q_reg[i] = s_tok.q[part * NK + i];
@@ -1028,7 +1056,7 @@ __global__ void __launch_bounds__(64) ffa_merge_splits_kernel(const DecodeParams
 // ---------------------------------------------------------------------------------------
 // One workgroup per (b,h): exact (p == 0) or pruned (p > 0) decode with LDS-staged scores.
 // Dynamic LDS: max((t/64 + 1)*64 scores, NW*64*X merge floats) * 4 bytes.
-template <typename T, int DH, int NW, bool BEAM>
+template <typename T, int DH, int NW, bool BEAM, bool XFORM>
 __global__ void __launch_bounds__(NW * 64) ffa_decode_wg_kernel(const DecodeParams P) {
     using G = Geo<T, DH>;
     constexpr int X = G::X, NCH = G::NCH, LPR = G::LPR, RPI = G::RPI, NVL = G::NVL, VG = G::VG;
@@ -1057,9 +1085,9 @@ __global__ void __launch_bounds__(NW * 64) ffa_decode_wg_kernel(const DecodePara
 
     const bool token_wave = wave == 0;
     uint4 q_reg[G::QREG];
-    const bool q_in_lds = setup_q<T, DH>(P, bh, bh - b * P.H, tlen, first, token_wave, s_tok, q_reg, lane);
+    const bool q_in_lds = setup_q<T, DH, XFORM>(P, bh, bh - b * P.H, tlen, first, token_wave, s_tok, q_reg, lane);
     TokenRegs tok;
-    if (token_wave) tok = token_load<T, DH>(P, bh, s_tok, lane);
+    if (token_wave) tok = token_load<T, DH, XFORM>(P, bh, s_tok, lane);
 
     const int ntiles = (tlen + kWave - 1) / kWave;   // tiles of cached keys
     const int nscore = (tlen / kWave + 1) * kWave;   // score slots: keys 0..tlen, padded to 64
@@ -1233,7 +1261,7 @@ __global__ void __launch_bounds__(NW * 64) ffa_decode_wg_kernel(const DecodePara
 // -- then streams only the V rows that survive (the new token's row, appended by pass 1, is
 // an ordinary row of the sample's own cache by then).  Weights are normalised globally, hence
 // the pieces' partial outputs simply add up (merged by the last piece to arrive).
-template <typename T, int DH, int NW, bool BEAM>
+template <typename T, int DH, int NW, bool BEAM, bool XFORM>
 __global__ void __launch_bounds__(NW * 64) ffa_scores_kernel(const DecodeParams P) {
     using G = Geo<T, DH>;
     constexpr int NCH = G::NCH;
@@ -1253,9 +1281,9 @@ __global__ void __launch_bounds__(NW * 64) ffa_scores_kernel(const DecodeParams 
 
     const bool token_wave = split == P.n_splits - 1 && wave == 0;
     uint4 q_reg[G::QREG];
-    const bool q_in_lds = setup_q<T, DH>(P, bh, bh - b * P.H, tlen, first, token_wave, s_tok, q_reg, lane);
+    const bool q_in_lds = setup_q<T, DH, XFORM>(P, bh, bh - b * P.H, tlen, first, token_wave, s_tok, q_reg, lane);
     TokenRegs tok;
-    if (token_wave) tok = token_load<T, DH>(P, bh, s_tok, lane);
+    if (token_wave) tok = token_load<T, DH, XFORM>(P, bh, s_tok, lane);
 
     const int ntiles = (tlen + kWave - 1) / kWave;
     const int tile_lo = max(split * P.tiles_per_split, first / kWave);
@@ -1484,17 +1512,18 @@ static inline int check_launch() {
     return hipGetLastError() == hipSuccess ? FFA_OK : FFA_ERR_LAUNCH;
 }
 
-template <typename T, int DH, int NW, bool BEAM>
+template <typename T, int DH, int NW, bool BEAM, bool XFORM>
 static int launch_split(const DecodeParams& P, hipStream_t st) {
     const int n_split_heads = P.bh_total - P.n_whole;
     const dim3 grid((unsigned)(P.n_whole + n_split_heads * P.n_splits));
-    hipLaunchKernelGGL((ffa_decode_split_kernel<T, DH, NW, BEAM>), grid, dim3((NW + 1) * 64), 0, st, P);
+    hipLaunchKernelGGL((ffa_decode_split_kernel<T, DH, NW, BEAM, XFORM>), grid, dim3((NW + 1) * 64), 0, st,
+                       HOT_PARAMS_OF(P), P);
     if (n_split_heads > 0 && P.n_splits > 1 && P.combine == FFA_COMBINE_KERNEL)
         hipLaunchKernelGGL((ffa_merge_splits_kernel<T, DH>), dim3((unsigned)n_split_heads), dim3(64), 0, st, P);
     return check_launch();
 }
 
-template <typename T, int DH, int NW, int TPK, bool BEAM>
+template <typename T, int DH, int NW, int TPK, bool BEAM, bool XFORM>
 static int launch_split_tpk(const DecodeParams& P, hipStream_t st) {
     using G = Geo<T, DH>;
     // Combinations whose tile fits one group of at most 8 K loads and 8 V loads.
@@ -1502,7 +1531,8 @@ static int launch_split_tpk(const DecodeParams& P, hipStream_t st) {
                   (kWave / TPK) / G::RPI <= 8) {
         const int n_split_heads = P.bh_total - P.n_whole;
         const dim3 grid((unsigned)(P.n_whole + n_split_heads * P.n_splits));
-        hipLaunchKernelGGL((ffa_decode_split_tpk_kernel<T, DH, NW, TPK, BEAM>), grid, dim3((NW + 1) * 64), 0, st, P);
+        hipLaunchKernelGGL((ffa_decode_split_tpk_kernel<T, DH, NW, TPK, BEAM, XFORM>), grid, dim3((NW + 1) * 64), 0, st,
+                           HOT_PARAMS_OF(P), P);
         if (n_split_heads > 0 && P.n_splits > 1 && P.combine == FFA_COMBINE_KERNEL)
             hipLaunchKernelGGL((ffa_merge_splits_kernel<T, DH>), dim3((unsigned)n_split_heads), dim3(64), 0, st, P);
         return check_launch();
@@ -1511,17 +1541,17 @@ static int launch_split_tpk(const DecodeParams& P, hipStream_t st) {
     }
 }
 
-template <typename T, int DH, int NW, bool BEAM>
+template <typename T, int DH, int NW, bool BEAM, bool XFORM>
 static int launch_two_pass(const DecodeParams& P, hipStream_t st) {
     const dim3 grid((unsigned)(P.bh_total * P.n_splits));
-    hipLaunchKernelGGL((ffa_scores_kernel<T, DH, NW, BEAM>), grid, dim3(NW * 64), 0, st, P);
+    hipLaunchKernelGGL((ffa_scores_kernel<T, DH, NW, BEAM, XFORM>), grid, dim3(NW * 64), 0, st, P);
     hipLaunchKernelGGL((ffa_pruned_pv_kernel<T, DH, NW, BEAM>), grid, dim3(NW * 64), 0, st, P);
     return check_launch();
 }
 
-template <typename T, int DH, int NW, bool BEAM>
+template <typename T, int DH, int NW, bool BEAM, bool XFORM>
 static int launch_wg(const DecodeParams& P, size_t lds_bytes, hipStream_t st) {
-    auto kern = ffa_decode_wg_kernel<T, DH, NW, BEAM>;
+    auto kern = ffa_decode_wg_kernel<T, DH, NW, BEAM, XFORM>;
     if (lds_bytes > 48 * 1024) {
         // Raise the dynamic-LDS ceiling once per instantiation and device (gfx950: 160 KiB per
         // CU).  The attribute is a property of the loaded function, not of a stream, so the
@@ -1545,7 +1575,7 @@ static int launch_wg(const DecodeParams& P, size_t lds_bytes, hipStream_t st) {
     return check_launch();
 }
 
-template <typename T, int DH, bool BEAM>
+template <typename T, int DH, bool BEAM, bool XFORM>
 static int dispatch_waves(const DecodeParams& P, const ffa_launch_plan& plan, hipStream_t st) {
     if (plan.kind == FFA_LAUNCH_SPLIT && plan.threads_per_key > 1) {
         if constexpr (DH == 80) {  // 10 / 20 chunks per key do not divide among 2 or 4 lanes
@@ -1553,64 +1583,64 @@ static int dispatch_waves(const DecodeParams& P, const ffa_launch_plan& plan, hi
         } else {
             const int key = plan.threads_per_key * 100 + plan.waves_per_wg;
             switch (key) {
-                case 204: return launch_split_tpk<T, DH, 4, 2, BEAM>(P, st);
-                case 208: return launch_split_tpk<T, DH, 8, 2, BEAM>(P, st);
-                case 404: return launch_split_tpk<T, DH, 4, 4, BEAM>(P, st);
-                case 408: return launch_split_tpk<T, DH, 8, 4, BEAM>(P, st);
+                case 204: return launch_split_tpk<T, DH, 4, 2, BEAM, XFORM>(P, st);
+                case 208: return launch_split_tpk<T, DH, 8, 2, BEAM, XFORM>(P, st);
+                case 404: return launch_split_tpk<T, DH, 4, 4, BEAM, XFORM>(P, st);
+                case 408: return launch_split_tpk<T, DH, 8, 4, BEAM, XFORM>(P, st);
                 default: return FFA_ERR_PLAN;
             }
         }
     }
     if (plan.kind == FFA_LAUNCH_SPLIT) {
         switch (plan.waves_per_wg) {
-            case 1: return launch_split<T, DH, 1, BEAM>(P, st);
-            case 2: return launch_split<T, DH, 2, BEAM>(P, st);
-            case 3: return launch_split<T, DH, 3, BEAM>(P, st);
-            case 4: return launch_split<T, DH, 4, BEAM>(P, st);
-            case 5: return launch_split<T, DH, 5, BEAM>(P, st);
-            case 6: return launch_split<T, DH, 6, BEAM>(P, st);
-            case 7: return launch_split<T, DH, 7, BEAM>(P, st);
-            case 8: return launch_split<T, DH, 8, BEAM>(P, st);
+            case 1: return launch_split<T, DH, 1, BEAM, XFORM>(P, st);
+            case 2: return launch_split<T, DH, 2, BEAM, XFORM>(P, st);
+            case 3: return launch_split<T, DH, 3, BEAM, XFORM>(P, st);
+            case 4: return launch_split<T, DH, 4, BEAM, XFORM>(P, st);
+            case 5: return launch_split<T, DH, 5, BEAM, XFORM>(P, st);
+            case 6: return launch_split<T, DH, 6, BEAM, XFORM>(P, st);
+            case 7: return launch_split<T, DH, 7, BEAM, XFORM>(P, st);
+            case 8: return launch_split<T, DH, 8, BEAM, XFORM>(P, st);
             default: return FFA_ERR_PLAN;
         }
     }
     if (plan.kind == FFA_LAUNCH_TWO_PASS) {
         switch (plan.waves_per_wg) {
-            case 1: return launch_two_pass<T, DH, 1, BEAM>(P, st);
-            case 2: return launch_two_pass<T, DH, 2, BEAM>(P, st);
-            case 4: return launch_two_pass<T, DH, 4, BEAM>(P, st);
-            case 8: return launch_two_pass<T, DH, 8, BEAM>(P, st);
+            case 1: return launch_two_pass<T, DH, 1, BEAM, XFORM>(P, st);
+            case 2: return launch_two_pass<T, DH, 2, BEAM, XFORM>(P, st);
+            case 4: return launch_two_pass<T, DH, 4, BEAM, XFORM>(P, st);
+            case 8: return launch_two_pass<T, DH, 8, BEAM, XFORM>(P, st);
             default: return FFA_ERR_PLAN;
         }
     }
     const size_t lds = wg_dynamic_lds_bytes(P.t, plan.waves_per_wg, (int)sizeof(T));
     switch (plan.waves_per_wg) {
-        case 1: return launch_wg<T, DH, 1, BEAM>(P, lds, st);
-        case 2: return launch_wg<T, DH, 2, BEAM>(P, lds, st);
-        case 4: return launch_wg<T, DH, 4, BEAM>(P, lds, st);
-        case 8: return launch_wg<T, DH, 8, BEAM>(P, lds, st);
-        case 16: return launch_wg<T, DH, 16, BEAM>(P, lds, st);
+        case 1: return launch_wg<T, DH, 1, BEAM, XFORM>(P, lds, st);
+        case 2: return launch_wg<T, DH, 2, BEAM, XFORM>(P, lds, st);
+        case 4: return launch_wg<T, DH, 4, BEAM, XFORM>(P, lds, st);
+        case 8: return launch_wg<T, DH, 8, BEAM, XFORM>(P, lds, st);
+        case 16: return launch_wg<T, DH, 16, BEAM, XFORM>(P, lds, st);
         default: return FFA_ERR_PLAN;
     }
 }
 
-template <typename T>
+template <typename T, bool XFORM>
 static int dispatch_head_dim(const DecodeParams& P, int head_dim, const ffa_launch_plan& plan,
                              hipStream_t st) {
     if (P.cache_indir != nullptr) {
         switch (head_dim) {
-            case 64: return dispatch_waves<T, 64, true>(P, plan, st);
-            case 80: return dispatch_waves<T, 80, true>(P, plan, st);
-            case 128: return dispatch_waves<T, 128, true>(P, plan, st);
-            case 256: return dispatch_waves<T, 256, true>(P, plan, st);
+            case 64: return dispatch_waves<T, 64, true, XFORM>(P, plan, st);
+            case 80: return dispatch_waves<T, 80, true, XFORM>(P, plan, st);
+            case 128: return dispatch_waves<T, 128, true, XFORM>(P, plan, st);
+            case 256: return dispatch_waves<T, 256, true, XFORM>(P, plan, st);
             default: return FFA_ERR_HEAD_DIM;
         }
     }
     switch (head_dim) {
-        case 64: return dispatch_waves<T, 64, false>(P, plan, st);
-        case 80: return dispatch_waves<T, 80, false>(P, plan, st);
-        case 128: return dispatch_waves<T, 128, false>(P, plan, st);
-        case 256: return dispatch_waves<T, 256, false>(P, plan, st);
+        case 64: return dispatch_waves<T, 64, false, XFORM>(P, plan, st);
+        case 80: return dispatch_waves<T, 80, false, XFORM>(P, plan, st);
+        case 128: return dispatch_waves<T, 128, false, XFORM>(P, plan, st);
+        case 256: return dispatch_waves<T, 256, false, XFORM>(P, plan, st);
         default: return FFA_ERR_HEAD_DIM;
     }
 }

@@ -151,12 +151,15 @@ int plan_launch_ex(int precision, int B, int H, int Dh, int t, float p, int use_
 int validate_plan(const ffa_launch_plan& plan, int precision, int head_dim, int bh, int t, float p);
 bool tpk_supported(int precision, int head_dim, int tpk);
 
-// launchers (ffa_kernels.hip; the decode kernels of each element type are a translation unit of
-// their own: ffa_decode_f16.hip, ffa_decode_bf16.hip, ffa_decode_f32.hip)
+// launchers (ffa_kernels.hip; the decode kernels of each element type, with and without the
+// transform of the new token, are a translation unit of their own: ffa_decode_<type>[_xform].hip)
 int launch_decode(const DecodeArgs& a, const ffa_launch_plan& plan, const WorkspaceView& ws);
 int launch_decode_f16(const DecodeParams& P, int head_dim, const ffa_launch_plan& plan, void* stream);
 int launch_decode_bf16(const DecodeParams& P, int head_dim, const ffa_launch_plan& plan, void* stream);
 int launch_decode_f32(const DecodeParams& P, int head_dim, const ffa_launch_plan& plan, void* stream);
+int launch_decode_f16_xform(const DecodeParams& P, int head_dim, const ffa_launch_plan& plan, void* stream);
+int launch_decode_bf16_xform(const DecodeParams& P, int head_dim, const ffa_launch_plan& plan, void* stream);
+int launch_decode_f32_xform(const DecodeParams& P, int head_dim, const ffa_launch_plan& plan, void* stream);
 constexpr int kMaxDevices = 64;
 int current_device();  // index of the current HIP device, -1 if none or beyond kMaxDevices
 int launch_init_cache(int precision, void* k_dst, void* v_dst, const void* k_src,

@@ -132,6 +132,12 @@ int launch_decode(const DecodeArgs& a, const ffa_launch_plan& plan, const Worksp
     P.rotary_dim = a.rotary_dim;
     P.xform = a.transforms_token() ? 1 : 0;
     P.rotary_coef = a.rotary_dim > 0 ? -2.0 * log2((double)a.rotary_base) / (double)a.rotary_dim : 0.0;
+    // The transform is a compile-time switch of the kernels: the plain step carries none of its code.
+    if (P.xform) {
+        if (a.precision == FFA_PRECISION_F16) return launch_decode_f16_xform(P, a.Dh, plan, a.stream);
+        if (a.precision == FFA_PRECISION_BF16) return launch_decode_bf16_xform(P, a.Dh, plan, a.stream);
+        return launch_decode_f32_xform(P, a.Dh, plan, a.stream);
+    }
     if (a.precision == FFA_PRECISION_F16) return launch_decode_f16(P, a.Dh, plan, a.stream);
     if (a.precision == FFA_PRECISION_BF16) return launch_decode_bf16(P, a.Dh, plan, a.stream);
     return launch_decode_f32(P, a.Dh, plan, a.stream);
