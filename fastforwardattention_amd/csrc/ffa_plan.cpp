@@ -231,13 +231,14 @@ int validate_plan(const ffa_launch_plan& plan, int precision, int head_dim, int 
             if (plan.whole_heads < 0 || plan.whole_heads > bh) return FFA_ERR_PLAN;
             if (plan.whole_heads < bh && (long long)plan.n_splits * plan.tiles_per_split < ntiles)
                 return FFA_ERR_PLAN;
-            if ((long long)(bh - plan.whole_heads) * plan.n_splits > 4 * kMaxSplitWorkgroups)
+            // Unsplit pairs are one workgroup each however many there are; the cap is on splitting.
+            if (plan.n_splits > 1 && (long long)(bh - plan.whole_heads) * plan.n_splits > 4 * kMaxSplitWorkgroups)
                 return FFA_ERR_PLAN;
             return FFA_OK;
         case FFA_LAUNCH_TWO_PASS:
             if (w > 8 || plan.whole_heads != 0 || plan.combine != FFA_COMBINE_FUSED) return FFA_ERR_PLAN;
             if ((long long)plan.n_splits * plan.tiles_per_split < ntiles) return FFA_ERR_PLAN;
-            if ((long long)bh * plan.n_splits > 4 * kMaxSplitWorkgroups) return FFA_ERR_PLAN;
+            if (plan.n_splits > 1 && (long long)bh * plan.n_splits > 4 * kMaxSplitWorkgroups) return FFA_ERR_PLAN;
             return FFA_OK;
         default:
             return FFA_ERR_PLAN;

@@ -25,7 +25,7 @@ def _say(*a):
 
 
 # ------------------------------------------------------------------ configs[2]: long sequences, B = 1
-@pytest.mark.parametrize("x", [1024, 4096, 16384])
+@pytest.mark.parametrize("x", [1024, 2048, 4096, 8192, 16384])
 @pytest.mark.parametrize("use_default", [False, True])
 def test_long_sequence_sweep_consecutive_steps(x, use_default):
     """BASELINE configs[2]: batch 1, 32 heads x 64, fp16, prompt x-128 of N(0,1), then decode
@@ -82,6 +82,56 @@ def test_opt13b_shape_small_batches(B):
         gk, gv = sess.caches()
         np.testing.assert_array_equal(gk.view(np.uint8), kc.view(np.uint8))
         np.testing.assert_array_equal(gv.view(np.uint8), vc.view(np.uint8))
+
+
+def test_opt13b_b10_whole_decode_at_the_reference_max_len():
+    """BASELINE configs[1] as the reference's script sizes it (example.py:29-35: prompt 1000,
+    max_len = 1000 + 128, so the chunk rows of K are 1128 x 16 bytes apart): B = 10, 32 heads x
+    64, fp16, all 128 decode steps in one session through the C ABI with the library's own
+    plans.  Every step is checked against the CPU oracle on two samples (64 of the 320 pairs);
+    their caches bit for bit at the end."""
+    B, H, Dh, prec, L, steps = 10, 32, 64, 16, 1000, 128
+    Lmax = L + steps
+    rng, K, V = rand_inputs(440, B, H, L, Dh, prec, kv_scale=0.5)
+    sess = CApiSession(K, V, Lmax)
+    sub = [0, 9]
+    kc, vc = O.pack_k_cache(K[sub], Lmax), O.pack_v_cache(V[sub], Lmax)
+    worst, kinds = 0.0, set()
+    for i in range(steps):
+        t = L + i
+        q, k, v = rand_token(rng, B, H, Dh, prec)
+        plan = capi.plan_launch(prec, B, H, Dh, t, 0.0, False)
+        kinds.add((plan.kind, plan.n_splits, plan.whole_heads))
+        if i % 32 == 0:
+            _say("opt1.3b b10 Lmax 1128", t, plan)
+        got = sess.step(q, k, v, 0.125, t)   # plan = NULL: what a caller of the reference's API gets
+        want = O.decode_step(q[sub], k[sub], v[sub], kc, vc, 0.125, t, acc=np.float64)
+        worst = max(worst, float(np.abs(got[sub] - want).max()))
+    assert worst <= TOL[prec], worst
+    assert all(kind == capi.FFA_LAUNCH_SPLIT and whole == 256 for kind, _, whole in kinds), kinds
+    gk, gv = sess.caches()
+    np.testing.assert_array_equal(gk[sub].view(np.uint16), kc.view(np.uint16))
+    np.testing.assert_array_equal(gv[sub].view(np.uint16), vc.view(np.uint16))
+
+
+def test_opt13b_shape_b2_last_step():
+    """BASELINE configs[1] at B = 2 (64 pairs, every pair cut into four pieces), last steps of the
+    256-step decode (t = 1253 .. 1255, max_len 1256), both launches."""
+    B, H, Dh, prec, L, Lmax = 2, 32, 64, 16, 1253, 1256
+    rng, K, V = rand_inputs(450, B, H, L, Dh, prec, kv_scale=0.5)
+    for use_default in (False, True):
+        sess = CApiSession(K, V, Lmax)
+        kc, vc = O.pack_k_cache(K, Lmax), O.pack_v_cache(V, Lmax)
+        for t in range(L, Lmax):
+            q, k, v = rand_token(rng, B, H, Dh, prec)
+            plan = capi.plan_launch(prec, B, H, Dh, t, 0.0, use_default)
+            _say("opt1.3b b2", use_default, t, plan)
+            got = sess.step(q, k, v, 0.125, t, plan=plan)
+            want = O.decode_step(q, k, v, kc, vc, 0.125, t, acc=np.float64)
+            assert float(np.abs(got - want).max()) <= TOL[prec]
+        gk, gv = sess.caches()
+        np.testing.assert_array_equal(gk.view(np.uint16), kc.view(np.uint16))
+        np.testing.assert_array_equal(gv.view(np.uint16), vc.view(np.uint16))
 
 
 # ------------------------------------------------------------------ configs[3]: GPT-J shape
