@@ -61,7 +61,6 @@ int run_decode(const DecodeArgs& args, const ffa_launch_plan* user_plan, void* w
     // words that persist from call to call; nothing else is ever placed on them.
     WorkspaceView ws = {nullptr, nullptr, nullptr, nullptr, 0};
     const int bh = a.B * a.H;
-    const int split_heads = bh - plan.whole_heads;
     const size_t need = plan_workspace_bytes(plan, bh, a.Dh, a.Lmax);
     if (need > 0) {
         if (workspace == nullptr || workspace_bytes < need) return FFA_ERR_WORKSPACE;
@@ -78,9 +77,7 @@ int run_decode(const DecodeArgs& args, const ffa_launch_plan* user_plan, void* w
             ws.scores = reinterpret_cast<float*>(base);
             ws.score_stride = score_stride_for(a.Lmax);
         } else {
-            ws.ml = reinterpret_cast<float*>(base);
-            ws.acc = reinterpret_cast<float*>(
-                base + align_up((size_t)split_heads * plan.n_splits * 2 * sizeof(float), 256));
+            ws.acc = reinterpret_cast<float*>(base);  // slots: accumulator, (max, sum), padding
         }
     }
     return launch_decode(a, plan, ws);
@@ -281,7 +278,7 @@ int ffa_attention_static_scratch(int precision, int batch_size, int head_num, in
         // The array keeps whatever the previous call on this GPU left behind: the arrival
         // counters of this call's pairs are cleared first (a small kernel, not a memset node,
         // so the call may be recorded into a HIP graph).
-        st = launch_fill_u32(static_cast<unsigned int*>(scratch_ptr), (size_t)a.B * a.H, 0u, stream);
+        st = launch_fill_u32(static_cast<unsigned int*>(scratch_ptr), (size_t)a.B * a.H * kCounterStride, 0u, stream);
         if (st != FFA_OK) return st;
     }
     return run_decode(a, &chosen, scratch_ptr, need > 0 ? kStaticScratchBytes : 0);

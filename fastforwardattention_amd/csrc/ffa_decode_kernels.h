@@ -602,9 +602,12 @@ __device__ __forceinline__ void finish_piece(const DecodeParams& P, int bh, int 
     }
 
     T* out = reinterpret_cast<T*>(P.out) + (size_t)bh * DH;
-    // Partials of split pairs: slot (bh - n_whole) of the workspace.
+    // Partials of split pairs: n_splits slots of the workspace per pair, each the accumulator
+    // followed by (max, sum) and padded to whole 256-byte lines, so that no two workgroups ever
+    // write into the same line.
+    constexpr int SLOT = DH + kSlotTailFloats;
     const size_t slot0 = (size_t)(bh - P.n_whole) * P.n_splits;
-    float* wa = P.ws_acc + (slot0 + split) * DH;
+    float* wa = P.ws_acc + (slot0 + split) * SLOT;
     for (int d = tid; d < DH; d += NOUT * 64) {
         float o = 0.f;
 #pragma unroll
@@ -617,9 +620,8 @@ __device__ __forceinline__ void finish_piece(const DecodeParams& P, int bh, int 
     if (P.combine != FFA_COMBINE_FUSED) {
         // A second kernel merges: plain stores would do, the kernel boundary publishes them.
         if (tid == 0) {
-            float* ml = P.ws_ml + (slot0 + split) * 2;
-            ml[0] = M;
-            ml[1] = L;
+            wa[DH] = M;
+            wa[DH + 1] = L;
         }
         return;
     }
@@ -635,14 +637,13 @@ __device__ __forceinline__ void finish_piece(const DecodeParams& P, int bh, int 
     // wave that sees the final count -- n_splits pieces x publishing waves -- knows that
     // every partial of the pair is in memory and merges all of them.
     if (tid == 0) {
-        float* ml = P.ws_ml + (slot0 + split) * 2;
-        publish(&ml[0], M);
-        publish(&ml[1], L);
+        publish(&wa[DH], M);
+        publish(&wa[DH + 1], L);
     }
     wait_published();
     unsigned prev = 0;
     if (lane == 0)
-        prev = __hip_atomic_fetch_add(&P.ws_cnt[bh], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        prev = __hip_atomic_fetch_add(&P.ws_cnt[(size_t)bh * kCounterStride], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     prev = __builtin_amdgcn_readfirstlane(prev);
     if (prev != (unsigned)(n_splits * NOUT - 1)) return;
     // Compiler-only barrier: the loads of the merge below must stay behind the counter
@@ -650,7 +651,7 @@ __device__ __forceinline__ void finish_piece(const DecodeParams& P, int bh, int 
     __atomic_signal_fence(__ATOMIC_SEQ_CST);
 
     // Merge: all loads of a batch of splits are issued before any is consumed.
-    const float* ml = P.ws_ml + slot0 * 2;
+    const float* pa = P.ws_acc + slot0 * SLOT;
     constexpr int MB = 8;
     for (int d = lane; d < DH; d += kWave) {
         float Mg = -INFINITY, o = 0.f, Lg = 0.f;
@@ -659,9 +660,9 @@ __device__ __forceinline__ void finish_piece(const DecodeParams& P, int bh, int 
 #pragma unroll
             for (int j = 0; j < MB; ++j) {
                 const int sj = min(s0 + j, n_splits - 1);
-                ms[j] = acquire(&ml[2 * sj]);
-                ls[j] = acquire(&ml[2 * sj + 1]);
-                as[j] = acquire(&P.ws_acc[(slot0 + sj) * DH + d]);
+                ms[j] = acquire(&pa[(size_t)sj * SLOT + DH]);
+                ls[j] = acquire(&pa[(size_t)sj * SLOT + DH + 1]);
+                as[j] = acquire(&pa[(size_t)sj * SLOT + d]);
             }
             float Mb = Mg;
 #pragma unroll
@@ -683,7 +684,7 @@ __device__ __forceinline__ void finish_piece(const DecodeParams& P, int bh, int 
         store_out(out, d, Lg > 0.f ? o / Lg : 0.f);
     }
     // Ready for the next launch on this stream (kernel boundaries order this store).
-    if (lane == 0) __hip_atomic_store(&P.ws_cnt[bh], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (lane == 0) __hip_atomic_store(&P.ws_cnt[(size_t)bh * kCounterStride], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 // ---------------------------------------------------------------------------------------
@@ -1036,18 +1037,18 @@ ffa_decode_split_tpk_kernel(HOT_PARAMS_DECL, const DecodeParams P_rest) {
 template <typename T, int DH>
 __global__ void __launch_bounds__(64) ffa_merge_splits_kernel(const DecodeParams P) {
     const int bh = P.n_whole + blockIdx.x, tid = threadIdx.x;
-    const size_t slot0 = (size_t)blockIdx.x * P.n_splits;
-    const float* ml = P.ws_ml + slot0 * 2;
+    constexpr int SLOT = DH + kSlotTailFloats;
+    const float* pa = P.ws_acc + (size_t)blockIdx.x * P.n_splits * SLOT;
     float Mg = -INFINITY;
-    for (int s = 0; s < P.n_splits; ++s) Mg = fmaxf(Mg, ml[2 * s]);
+    for (int s = 0; s < P.n_splits; ++s) Mg = fmaxf(Mg, pa[(size_t)s * SLOT + DH]);
     T* out = reinterpret_cast<T*>(P.out) + (size_t)bh * DH;
     for (int d = tid; d < DH; d += 64) {
         float o = 0.f, Lg = 0.f;
         for (int s = 0; s < P.n_splits; ++s) {
-            const float ms = ml[2 * s];
+            const float ms = pa[(size_t)s * SLOT + DH];
             const float w = (ms == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(ms - Mg);
-            Lg += w * ml[2 * s + 1];
-            o += w * P.ws_acc[(slot0 + s) * DH + d];
+            Lg += w * pa[(size_t)s * SLOT + DH + 1];
+            o += w * pa[(size_t)s * SLOT + d];
         }
         store_out(out, d, Lg > 0.f ? o / Lg : 0.f);
     }
@@ -1484,7 +1485,7 @@ __global__ void __launch_bounds__(NW * 64) ffa_pruned_pv_kernel(const DecodePara
     wait_published();
     unsigned prev = 0;
     if (lane == 0)
-        prev = __hip_atomic_fetch_add(&P.ws_cnt[bh], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        prev = __hip_atomic_fetch_add(&P.ws_cnt[(size_t)bh * kCounterStride], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     prev = __builtin_amdgcn_readfirstlane(prev);
     if (prev != (unsigned)(P.n_splits * NPUB - 1)) return;
     __atomic_signal_fence(__ATOMIC_SEQ_CST);  // compiler-only: keep the merge loads behind the counter
@@ -1503,7 +1504,7 @@ __global__ void __launch_bounds__(NW * 64) ffa_pruned_pv_kernel(const DecodePara
         }
         store_out(out, d, all_masked ? 0.f : o);
     }
-    if (lane == 0) __hip_atomic_store(&P.ws_cnt[bh], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (lane == 0) __hip_atomic_store(&P.ws_cnt[(size_t)bh * kCounterStride], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 // ---------------------------------------------------------------------------------------

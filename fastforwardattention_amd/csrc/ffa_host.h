@@ -55,9 +55,9 @@ struct DecodeParams {
     void* v_cache;
     void* out;
     const int* seq_lengths;
-    float* ws_acc;         // [BH, n_splits, Dh]
-    float* ws_ml;          // [BH, n_splits, 2]
-    unsigned int* ws_cnt;  // [BH]
+    float* ws_acc;         // split launch: [split pairs, n_splits, Dh + kSlotTailFloats]; two-pass: [BH, n_splits, Dh]
+    float* ws_ml;          // two-pass: [BH, n_splits, 2]
+    unsigned int* ws_cnt;  // [BH] arrival counters, kCounterStride words apart
     float* ws_scores;      // [BH, score_stride] raw q.k of the two-pass path
     int score_stride;      // floats per (b,h) row of ws_scores, a multiple of 64
     unsigned int* kept_count;
@@ -83,8 +83,8 @@ struct DecodeParams {
 // Carved-up workspace for a given plan.
 struct WorkspaceView {
     unsigned int* cnt;  // [B*H] arrival counters, zero between launches
-    float* ml;          // [split pairs, n_splits, 2]
-    float* acc;         // [split pairs, n_splits, Dh]
+    float* ml;          // two-pass: [B*H, n_splits, 2] piece (max, sum)
+    float* acc;         // split: [split pairs, n_splits, Dh + kSlotTailFloats]; two-pass: [B*H, n_splits, Dh]
     float* scores;      // two-pass path: [B*H, score_stride] raw scores
     int score_stride;
 };
@@ -111,13 +111,19 @@ inline int max_splits_for(int bh, int max_seq_len) {
     return m < 1 ? 1 : m;
 }
 
-inline size_t workspace_counter_bytes(int bh) { return align_up((size_t)bh * sizeof(unsigned int), 256); }
+// Arrival counters sit kCounterStride words apart: one per 256 bytes, so that the read-modify-writes
+// of different (batch, head) pairs, which arrive in bursts, do not queue up on one cache line.
+constexpr int kCounterStride = 64;
+inline size_t workspace_counter_bytes(int bh) { return (size_t)bh * kCounterStride * sizeof(unsigned int); }
 
-// bh = all (batch, head) pairs (counter array), split_heads = pairs that are split.
+// A partial of the exact split launch: accumulator [Dh], then (max, sum), padded to whole 256-byte
+// lines so that workgroups never write into each other's lines.
+constexpr int kSlotTailFloats = 64;
+// bh = all (batch, head) pairs (counter array), split_heads = pairs that are split:
+// [counters][split_heads x n_splits slots].
 inline size_t workspace_bytes_for(int bh, int split_heads, int head_dim, int n_splits) {
     if (n_splits <= 1 || split_heads <= 0) return workspace_counter_bytes(bh);
-    return workspace_counter_bytes(bh) + align_up((size_t)split_heads * n_splits * 2 * sizeof(float), 256) +
-           (size_t)split_heads * n_splits * head_dim * sizeof(float);
+    return workspace_counter_bytes(bh) + (size_t)split_heads * n_splits * (head_dim + kSlotTailFloats) * sizeof(float);
 }
 
 // Two-pass path: counters, piece (max, sum) [bh, n_splits, 2], partial outputs

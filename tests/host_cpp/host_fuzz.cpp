@@ -68,16 +68,14 @@ int launch_decode(const DecodeArgs& a, const ffa_launch_plan& plan, const Worksp
         CHECK(split_heads >= 0);
         if (plan.n_splits > 1 && split_heads > 0) {
             const size_t slots = (size_t)split_heads * plan.n_splits;
-            inside(ws.cnt, (size_t)bh * 4);
-            inside(ws.ml, slots * 2 * 4);
-            inside(ws.acc, slots * a.Dh * 4);
-            CHECK(reinterpret_cast<const char*>(ws.ml) >= reinterpret_cast<const char*>(ws.cnt) + (size_t)bh * 4);
-            CHECK(reinterpret_cast<const char*>(ws.acc) >= reinterpret_cast<const char*>(ws.ml) + slots * 8);
+            inside(ws.cnt, (size_t)bh * kCounterStride * 4);
+            inside(ws.acc, slots * (a.Dh + kSlotTailFloats) * 4);
+            CHECK(reinterpret_cast<const char*>(ws.acc) >= reinterpret_cast<const char*>(ws.cnt) + (size_t)bh * kCounterStride * 4);
             CHECK((long long)plan.n_splits * plan.tiles_per_split >= num_tiles(a.t));
         }
     } else if (plan.kind == FFA_LAUNCH_TWO_PASS) {
         const size_t slots = (size_t)bh * plan.n_splits;
-        inside(ws.cnt, (size_t)bh * 4);
+        inside(ws.cnt, (size_t)bh * kCounterStride * 4);
         inside(ws.ml, slots * 2 * 4);
         inside(ws.acc, slots * a.Dh * 4);
         CHECK(ws.score_stride >= a.t + 1 && ws.score_stride % 64 == 0);
