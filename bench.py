@@ -460,15 +460,24 @@ class PrunedWorkload:
         return plan
 
     def run(self, p, steps=320, warmup=8):
+        # Timed as replays of a HIP graph holding the `steps` launches, like the headline: at
+        # B = 1 a pruned step is two short kernels and eager launches from Python cannot keep up.
         torch = self.torch
-        sp = torch.cuda.current_stream().cuda_stream
-        for i in range(warmup):
-            plan = self.launch(i, p, sp)
-
-        def body():
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            for i in range(warmup):
+                plan = self.launch(i, p, side.cuda_stream)
+        side.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=side):
+            sp = torch.cuda.current_stream().cuda_stream
             for i in range(steps):
                 self.launch(i, p, sp)
-        ms = time_region(torch, body)
+        graph.replay()
+        torch.cuda.synchronize()
+        ms = median([time_region(torch, graph.replay) for _ in range(3)])
+        sp = torch.cuda.current_stream().cuda_stream
         out_p = self.out.clone()
         # skip fraction at the last step (diagnostic launch, untimed)
         self.launch(steps - 1, p, sp, diag=True)
@@ -736,13 +745,13 @@ class SweepShape:
         torch.cuda.synchronize()
 
     def time_plan(self, plan, t, region_ms=4.0, repeats=3):
-        """us per launch of `plan` at t cached keys: eager launches on rotating caches, best of
-        `repeats` regions of about `region_ms`.  None if the library refuses the plan."""
+        """us per launch of `plan` at t cached keys: launches on rotating caches recorded into a HIP
+        graph of about `region_ms` and replayed, best of `repeats` replays (eager launches from
+        Python cannot keep up with the short steps).  None if the library refuses the plan."""
         torch = self.torch
-        sp = torch.cuda.current_stream().cuda_stream
         scale = self.Dh ** -0.5
 
-        def go(n):
+        def go(n, sp):
             for i in range(n):
                 l = i % self.layers
                 rc = self.fn(self.B, self.H, self.Dh, self.Lmax, scale, t, self.q.data_ptr(), self.k.data_ptr(),
@@ -751,13 +760,25 @@ class SweepShape:
                 if rc != 0:
                     return rc
             return 0
-        if go(self.layers) != 0:
-            torch.cuda.synchronize()
-            return None
+        if not hasattr(self, "side"):
+            self.side = torch.cuda.Stream()
+        side = self.side
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            rc = go(self.layers, side.cuda_stream)
+            side.synchronize()
+            if rc != 0:
+                return None
+            ms = time_region(torch, lambda: go(2 * self.layers, side.cuda_stream))   # upper bound: eager
+        n = max(2 * self.layers, min(4000, int(region_ms / (ms / (2 * self.layers)))))
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=side):
+            go(n, torch.cuda.current_stream().cuda_stream)
+        graph.replay()
         torch.cuda.synchronize()
-        ms = time_region(torch, lambda: go(2 * self.layers))
-        n = max(2 * self.layers, int(region_ms / (ms / (2 * self.layers))))
-        return min(time_region(torch, lambda: go(n)) for _ in range(repeats)) * 1e3 / n
+        best = min(time_region(torch, graph.replay) for _ in range(repeats)) * 1e3 / n
+        del graph
+        return best
 
 
 def candidate_plans(capi, prec, B, H, Dh, t, p, cus):
@@ -791,19 +812,20 @@ def candidate_plans(capi, prec, B, H, Dh, t, p, cus):
                 geos += [(whole, base), (whole, 2 * base), (whole, max(1, base // 2))]
             geos.append((bh, 1))
         else:
-            geos += [(0, cus // bh), (0, max(1, cus // (2 * bh))), (0, 2 * cus // bh), (bh, 1)]
-        rule = out[0][1]
+            geos += [(0, cus // bh), (0, max(1, cus // (2 * bh))), (0, max(1, cus // (4 * bh))), (0, 2 * cus // bh), (bh, 1)]
+        lanes = [1] + [k for k in ((4,) if nch >= 16 else (2, 4)) if tpk_ok(k)]
         for w in (4, 8):
             for whole, ns in geos:
                 ns, tps = cut(ns)
-                out.append((f"split w{w} whole{whole} x{ns}",
-                            capi.make_plan(capi.FFA_LAUNCH_SPLIT, w, ns, tps, 0, bh if ns == 1 else whole)))
-            if rule.kind == capi.FFA_LAUNCH_SPLIT:
-                for k in (2, 4):
-                    if tpk_ok(k):
-                        out.append((f"split w{w} lanes/key {k} whole{rule.whole_heads} x{rule.n_splits}",
-                                    capi.make_plan(capi.FFA_LAUNCH_SPLIT, w, rule.n_splits, rule.tiles_per_split, 0,
-                                                   rule.whole_heads, threads_per_key=k)))
+                for k in lanes:
+                    out.append((f"split w{w}{f' lanes/key {k}' if k > 1 else ''} whole{bh if ns == 1 else whole} x{ns}",
+                                capi.make_plan(capi.FFA_LAUNCH_SPLIT, w, ns, tps, 0, bh if ns == 1 else whole,
+                                               threads_per_key=k)))
+        if bh < cus and ntiles <= 16:      # short sequences: also workgroups of two waves
+            for whole, ns in geos:
+                ns, tps = cut(ns)
+                out.append((f"split w2 whole{bh if ns == 1 else whole} x{ns}",
+                            capi.make_plan(capi.FFA_LAUNCH_SPLIT, 2, ns, tps, 0, bh if ns == 1 else whole)))
         if fits_lds:
             out += [(f"workgroup w{w}", capi.make_plan(capi.FFA_LAUNCH_WORKGROUP, w, 1, ntiles)) for w in (4, 8, 16)]
     seen, uniq = set(), []
@@ -814,16 +836,35 @@ def candidate_plans(capi, prec, B, H, Dh, t, p, cus):
     return uniq
 
 
-def run_plan_sweep(out_path):
+GRID_T = (128, 256, 512, 1024, 2048, 4096, 8192, 16384)
+GRID_BH = ((1, 16), (1, 32), (2, 32), (4, 32), (8, 32), (10, 32), (16, 32), (32, 32))
+
+
+def grid_shapes():
+    """The grid behind csrc/ffa_plan_grid.inc: pairs x head dim x length x pruned or not, away
+    from the BASELINE shapes, so that any problem finds a measured neighbour."""
+    out = []
+    for prec, dhs in ((16, (64, 128, 256)), (32, (64, 128))):
+        for Dh in dhs:
+            for B, H in GRID_BH:
+                for p in (0.0, 1e-2):
+                    out.append((prec, B, H, Dh, p, GRID_T[-1] + 64, list(GRID_T)))
+    return out
+
+
+def run_plan_sweep(out_path, grid=False, part=(0, 1)):
     """Times every candidate at every sweep point, prints one JSON line per point and writes the
     table.  A point keeps the rules' plan unless a candidate beats it by more than 3 % in a
-    second, longer timing of the two."""
+    second, longer timing of the two.  grid: the shapes of grid_shapes() (shape i belongs to part
+    i % parts) and rows keyed by their own (pairs, t), which the planner matches by nearest
+    neighbour; otherwise the BASELINE shapes and rows keyed by a range of t."""
     import torch
     from fastforwardattention_amd import capi
     lib = capi.load()
     cus = lib.ffa_device_compute_units()
     rows = []
-    for prec, B, H, Dh, p, max_len, ts in SWEEP_SHAPES:
+    shapes = [sh for i, sh in enumerate(grid_shapes()) if i % part[1] == part[0]] if grid else SWEEP_SHAPES
+    for prec, B, H, Dh, p, max_len, ts in shapes:
         shape = SweepShape(prec, B, H, Dh, p, max_len)
         for i, t in enumerate(ts):
             timed = []
@@ -845,6 +886,8 @@ def run_plan_sweep(out_path):
             # the point stands for the t halfway to its neighbours (an eighth beyond the ends)
             lo = (ts[i - 1] + t) // 2 + 1 if i > 0 else (t - (ts[1] - t) // 2 if len(ts) > 1 else t * 7 // 8)
             hi = (t + ts[i + 1]) // 2 if i + 1 < len(ts) else (t + (t - ts[i - 1]) // 2 if len(ts) > 1 else t * 9 // 8)
+            if grid:
+                lo = hi = t
             rows.append((prec, Dh, B * H, max(lo, 0), hi, 1 if p > 0 else 0, chosen, chosen_us, best_us, rule_us,
                          0 if chosen_label == "rules" else 1))
             print(json.dumps({"sweep_point": {"precision": prec, "B": B, "H": H, "Dh": Dh, "max_len": max_len, "t": t, "p": p},
@@ -854,23 +897,41 @@ def run_plan_sweep(out_path):
         del shape
         torch.cuda.empty_cache()
     dev = torch.cuda.get_device_name(0)
-    lines = [
-        "// Launch-plan table: measured choices that override the planner's rules at the points where a",
-        "// sweep on the device found a faster launch.  GENERATED -- do not edit by hand.",
-        "//   command : python bench.py --sweep-plans      (then rebuild the library)",
-        f"//   device  : {dev}, {cus} compute units",
-        "// Row: FFA_PLAN_ROW(override, precision, head_dim, pairs, t_lo, t_hi, pruned, kind, waves,",
-        "//                   threads_per_key, n_splits, whole_heads, chosen_us, best_us, rule_us)",
-        "//   override = 1: the planner launches this row's plan for t_lo <= t <= t_hi on a 256-CU device;",
-        "//   override = 0: the rules' own plan stayed within 3 % of the fastest candidate and is kept (the",
-        "//   row records the measurement).  pairs = batch * heads; pruned = 1 for prob_thresh > 0;",
-        "//   chosen_us is the time of the row's plan, best_us the fastest candidate of the sweep, rule_us",
-        "//   the time of what the rules alone launch.",
-    ]
-    for prec, Dh, pairs, lo, hi, pruned, plan, chosen_us, best_us, rule_us, override in rows:
-        lines.append(f"FFA_PLAN_ROW({override}, {prec}, {Dh}, {pairs}, {lo}, {hi}, {pruned}, {plan.kind}, "
-                     f"{plan.waves_per_wg}, {plan.threads_per_key}, {plan.n_splits}, {plan.whole_heads}, "
-                     f"{chosen_us:.2f}f, {best_us:.2f}f, {rule_us:.2f}f)")
+    if grid:
+        lines = [
+            "// Launch-plan grid: what a sweep on the device found fastest on a grid of problem sizes.  The",
+            "// planner looks up the nearest row (same precision, head dimension and pruned / exact; pairs and",
+            "// length each within a factor of sqrt 2) and, where the row overrides the rules, launches its",
+            "// kind, waves and lanes per key with the row's workgroup count re-cut for the actual problem.",
+            "// GENERATED -- do not edit by hand.",
+            "//   command : python bench.py --sweep-plans grid      (then rebuild the library)",
+            f"//   device  : {dev}, {cus} compute units",
+            "// Row: FFA_GRID_ROW(override, precision, head_dim, pairs, t, pruned, kind, waves, threads_per_key,",
+            "//                   n_splits, whole_heads, chosen_us, best_us, rule_us)",
+            "//   override = 0: the rules' own plan stayed within 3 % of the fastest candidate and is kept.",
+        ] if part[0] == 0 else []
+        for prec, Dh, pairs, lo, hi, pruned, plan, chosen_us, best_us, rule_us, override in rows:
+            lines.append(f"FFA_GRID_ROW({override}, {prec}, {Dh}, {pairs}, {lo}, {pruned}, {plan.kind}, "
+                         f"{plan.waves_per_wg}, {plan.threads_per_key}, {plan.n_splits}, {plan.whole_heads}, "
+                         f"{chosen_us:.2f}f, {best_us:.2f}f, {rule_us:.2f}f)")
+    else:
+        lines = [
+            "// Launch-plan table: measured choices that override the planner's rules at the points where a",
+            "// sweep on the device found a faster launch.  GENERATED -- do not edit by hand.",
+            "//   command : python bench.py --sweep-plans      (then rebuild the library)",
+            f"//   device  : {dev}, {cus} compute units",
+            "// Row: FFA_PLAN_ROW(override, precision, head_dim, pairs, t_lo, t_hi, pruned, kind, waves,",
+            "//                   threads_per_key, n_splits, whole_heads, chosen_us, best_us, rule_us)",
+            "//   override = 1: the planner launches this row's plan for t_lo <= t <= t_hi on a 256-CU device;",
+            "//   override = 0: the rules' own plan stayed within 3 % of the fastest candidate and is kept (the",
+            "//   row records the measurement).  pairs = batch * heads; pruned = 1 for prob_thresh > 0;",
+            "//   chosen_us is the time of the row's plan, best_us the fastest candidate of the sweep, rule_us",
+            "//   the time of what the rules alone launch.",
+        ]
+        for prec, Dh, pairs, lo, hi, pruned, plan, chosen_us, best_us, rule_us, override in rows:
+            lines.append(f"FFA_PLAN_ROW({override}, {prec}, {Dh}, {pairs}, {lo}, {hi}, {pruned}, {plan.kind}, "
+                         f"{plan.waves_per_wg}, {plan.threads_per_key}, {plan.n_splits}, {plan.whole_heads}, "
+                         f"{chosen_us:.2f}f, {best_us:.2f}f, {rule_us:.2f}f)")
     with open(out_path, "w") as f:
         f.write("\n".join(lines) + "\n")
     print(json.dumps({"plan_table": out_path, "rows": len(rows),
@@ -878,6 +939,7 @@ def run_plan_sweep(out_path):
 
 
 DEFAULT_SWEEP_OUT = os.path.join(ROOT, "fastforwardattention_amd", "csrc", "ffa_plan_table.inc")
+DEFAULT_GRID_OUT = os.path.join(ROOT, "fastforwardattention_amd", "csrc", "ffa_plan_grid.inc")
 
 
 def run_copy_calibration(mib=128, reps=40):
@@ -933,10 +995,12 @@ def main():
     ap.add_argument("--suite", action="store_true",
                     help="run every BASELINE configuration (tuned and default launch) and the pruned sweep; "
                          "one JSON line each instead of the single headline line")
-    ap.add_argument("--sweep-plans", action="store_true",
-                    help="time candidate launch plans at the BASELINE shapes and write the planner's table of "
-                         "overrides (then rebuild the library)")
-    ap.add_argument("--sweep-out", default=DEFAULT_SWEEP_OUT, help="where --sweep-plans writes the table")
+    ap.add_argument("--sweep-plans", nargs="?", const="baseline", default=None, metavar="baseline|grid[:i/n]",
+                    help="time candidate launch plans and write a table the planner compiles in (then rebuild the "
+                         "library): 'baseline' (default) = the BASELINE shapes -> csrc/ffa_plan_table.inc; 'grid' = a "
+                         "grid of problem sizes -> csrc/ffa_plan_grid.inc ('grid:i/n' = every n-th shape from the "
+                         "i-th, rows to be concatenated in order of i)")
+    ap.add_argument("--sweep-out", default=None, help="where --sweep-plans writes the table")
     ap.add_argument("--init-cache", action="store_true", help="only the cache-construction kernel at the BASELINE shapes")
     ap.add_argument("--pruned-sweep", action="store_true", help="only the pruned sweep (BASELINE configs[4])")
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -962,7 +1026,11 @@ def main():
         run_suite(args)
         return
     if args.sweep_plans:
-        run_plan_sweep(args.sweep_out)
+        if args.sweep_plans.startswith("grid"):
+            part = tuple(int(x) for x in args.sweep_plans.split(":")[1].split("/")) if ":" in args.sweep_plans else (0, 1)
+            run_plan_sweep(args.sweep_out or DEFAULT_GRID_OUT, grid=True, part=part)
+        else:
+            run_plan_sweep(args.sweep_out or DEFAULT_SWEEP_OUT)
         return
     if args.pruned_sweep:
         run_pruned_sweeps()

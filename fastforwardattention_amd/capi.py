@@ -71,6 +71,7 @@ SIGNATURES = {
     "ffa_device_compute_units": (_i, []),
     "ffa_plan_launch": (_i, [_i, _i, _i, _i, _i, _f, _i, _i, _PLAN_P]),
     "ffa_plan_launch_rules": (_i, [_i, _i, _i, _i, _i, _f, _i, _i, _PLAN_P]),
+    "ffa_plan_source": (_i, [_i, _i, _i, _i, _i, _f, _i]),
     "ffa_workspace_bytes": (_sz, [_i, _i, _i, _i]),
     "ffa_workspace_init": (_i, [_vp, _sz, _vp]),
     "ffa_init_cache_f16": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp]),

@@ -164,6 +164,15 @@ int ffa_plan_launch_rules(int precision, int batch_size, int head_num, int head_
                       use_default_kernel_launch, compute_units, /*use_table=*/0, plan);
 }
 
+int ffa_plan_source(int precision, int batch_size, int head_num, int head_dim, int t, float prob_thresh,
+                    int compute_units) {
+    ffa_launch_plan plan;
+    const int st = plan_entry(precision, batch_size, head_num, head_dim, t, prob_thresh, 0, compute_units, 1, &plan);
+    if (st != FFA_OK) return -st;
+    if (compute_units <= 0) compute_units = query_compute_units();
+    return plan_source(planner_precision(precision), batch_size, head_num, head_dim, t, prob_thresh, compute_units);
+}
+
 size_t ffa_workspace_bytes(int batch_size, int head_num, int head_dim, int max_seq_len) {
     if (batch_size <= 0 || head_num <= 0 || head_dim <= 0 || max_seq_len <= 0) return 0;
     const int bh = batch_size * head_num;

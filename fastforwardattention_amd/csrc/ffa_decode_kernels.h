@@ -65,6 +65,25 @@ __device__ __forceinline__ DecodeParams with_hot_params(const DecodeParams& rest
     return P;
 }
 
+// The same for the second kernel of the two-pass path, whose first loads are the pieces' (max, sum)
+// and the scores.
+#define PV_HOT_PARAMS_DECL                                                                                   \
+    float *hot_scores, float *hot_ml, void *hot_v_cache, const int *hot_seq_lengths, int hot_score_stride, \
+        int hot_Lmax, int hot_t, int hot_n_splits, unsigned hot_split_magic, int hot_tiles_per_split
+#define PV_HOT_PARAMS_USE                                                                                \
+    hot_scores, hot_ml, hot_v_cache, hot_seq_lengths, hot_score_stride, hot_Lmax, hot_t, hot_n_splits, \
+        hot_split_magic, hot_tiles_per_split
+#define PV_HOT_PARAMS_OF(P)                                                                              \
+    (P).ws_scores, (P).ws_ml, (P).v_cache, (P).seq_lengths, (P).score_stride, (P).Lmax, (P).t, (P).n_splits, \
+        (P).split_magic, (P).tiles_per_split
+__device__ __forceinline__ DecodeParams with_pv_hot_params(const DecodeParams& rest, PV_HOT_PARAMS_DECL) {
+    DecodeParams P = rest;
+    P.ws_scores = hot_scores; P.ws_ml = hot_ml; P.v_cache = hot_v_cache; P.seq_lengths = hot_seq_lengths;
+    P.score_stride = hot_score_stride; P.Lmax = hot_Lmax; P.t = hot_t; P.n_splits = hot_n_splits;
+    P.split_magic = hot_split_magic; P.tiles_per_split = hot_tiles_per_split;
+    return P;
+}
+
 // Per-(b) bounds, attention.cu:805-817.  tlen = slot of the new token = number of cached
 // keys; first = first unmasked key.  Values are clamped so that a bad seq_lengths entry
 // can never produce an out-of-bounds access.
@@ -1058,7 +1077,8 @@ __global__ void __launch_bounds__(64) ffa_merge_splits_kernel(const DecodeParams
 // One workgroup per (b,h): exact (p == 0) or pruned (p > 0) decode with LDS-staged scores.
 // Dynamic LDS: max((t/64 + 1)*64 scores, NW*64*X merge floats) * 4 bytes.
 template <typename T, int DH, int NW, bool BEAM, bool XFORM>
-__global__ void __launch_bounds__(NW * 64) ffa_decode_wg_kernel(const DecodeParams P) {
+__global__ void __launch_bounds__(NW * 64) ffa_decode_wg_kernel(HOT_PARAMS_DECL, const DecodeParams P_rest) {
+    const DecodeParams P = with_hot_params(P_rest, HOT_PARAMS_USE);
     using G = Geo<T, DH>;
     constexpr int X = G::X, NCH = G::NCH, LPR = G::LPR, RPI = G::RPI, NVL = G::NVL, VG = G::VG;
     constexpr int NT = NW * 64;
@@ -1263,7 +1283,8 @@ __global__ void __launch_bounds__(NW * 64) ffa_decode_wg_kernel(const DecodePara
 // an ordinary row of the sample's own cache by then).  Weights are normalised globally, hence
 // the pieces' partial outputs simply add up (merged by the last piece to arrive).
 template <typename T, int DH, int NW, bool BEAM, bool XFORM>
-__global__ void __launch_bounds__(NW * 64) ffa_scores_kernel(const DecodeParams P) {
+__global__ void __launch_bounds__(NW * 64) ffa_scores_kernel(HOT_PARAMS_DECL, const DecodeParams P_rest) {
+    const DecodeParams P = with_hot_params(P_rest, HOT_PARAMS_USE);
     using G = Geo<T, DH>;
     constexpr int NCH = G::NCH;
     __shared__ float s_m[NW], s_l[NW];
@@ -1352,7 +1373,8 @@ __global__ void __launch_bounds__(NW * 64) ffa_scores_kernel(const DecodeParams 
 }
 
 template <typename T, int DH, int NW, bool BEAM>
-__global__ void __launch_bounds__(NW * 64) ffa_pruned_pv_kernel(const DecodeParams P) {
+__global__ void __launch_bounds__(NW * 64) ffa_pruned_pv_kernel(PV_HOT_PARAMS_DECL, const DecodeParams P_rest) {
+    const DecodeParams P = with_pv_hot_params(P_rest, PV_HOT_PARAMS_USE);
     using G = Geo<T, DH>;
     constexpr int X = G::X, LPR = G::LPR;
     constexpr int NT = NW * 64;
@@ -1545,8 +1567,8 @@ static int launch_split_tpk(const DecodeParams& P, hipStream_t st) {
 template <typename T, int DH, int NW, bool BEAM, bool XFORM>
 static int launch_two_pass(const DecodeParams& P, hipStream_t st) {
     const dim3 grid((unsigned)(P.bh_total * P.n_splits));
-    hipLaunchKernelGGL((ffa_scores_kernel<T, DH, NW, BEAM, XFORM>), grid, dim3(NW * 64), 0, st, P);
-    hipLaunchKernelGGL((ffa_pruned_pv_kernel<T, DH, NW, BEAM>), grid, dim3(NW * 64), 0, st, P);
+    hipLaunchKernelGGL((ffa_scores_kernel<T, DH, NW, BEAM, XFORM>), grid, dim3(NW * 64), 0, st, HOT_PARAMS_OF(P), P);
+    hipLaunchKernelGGL((ffa_pruned_pv_kernel<T, DH, NW, BEAM>), grid, dim3(NW * 64), 0, st, PV_HOT_PARAMS_OF(P), P);
     return check_launch();
 }
 
@@ -1572,7 +1594,7 @@ static int launch_wg(const DecodeParams& P, size_t lds_bytes, hipStream_t st) {
             raised[dev] = true;
         }
     }
-    hipLaunchKernelGGL(kern, dim3((unsigned)P.bh_total), dim3(NW * 64), lds_bytes, st, P);
+    hipLaunchKernelGGL(kern, dim3((unsigned)P.bh_total), dim3(NW * 64), lds_bytes, st, HOT_PARAMS_OF(P), P);
     return check_launch();
 }
 

@@ -155,6 +155,9 @@ int plan_launch(int precision, int B, int H, int Dh, int t, float p, int use_def
 int plan_launch_ex(int precision, int B, int H, int Dh, int t, float p, int use_default, int cus,
                    int use_table, ffa_launch_plan* plan);
 int validate_plan(const ffa_launch_plan& plan, int precision, int head_dim, int bh, int t, float p);
+// Where the tuned plan of a problem comes from: 0 = the rules, 1 = a row of the table of the
+// BASELINE shapes, 2 = the nearest row of the grid.
+int plan_source(int precision, int B, int H, int Dh, int t, float p, int cus);
 bool tpk_supported(int precision, int head_dim, int tpk);
 
 // launchers (ffa_kernels.hip; the decode kernels of each element type, with and without the

@@ -7,6 +7,7 @@
 // the quantities that matter are how many wavefronts share a (batch, head) and how the
 // sequence is split across workgroups.
 #include <math.h>
+#include <stdlib.h>
 
 #include "ffa_host.h"
 
@@ -43,7 +44,9 @@ static int wg_waves_for(int ntiles, int want) {
 // ---------------------------------------------------------------------------------------
 // Measured overrides (ffa_plan_table.inc, written by `python bench.py --sweep-plans` on the
 // device): where a sweep over launch kinds, wave counts, lanes per key and split factors
-// found something more than 3 % faster than the rules below, the table's row wins.
+// found something more than 3 % faster than the rules below, the table's row wins.  The table
+// holds the BASELINE shapes themselves and matches them exactly; the grid further down covers
+// everything else by nearest neighbour.
 struct PlanRow {
     int override_rules, precision, head_dim, pairs, t_lo, t_hi, pruned;
     int kind, waves, tpk, n_splits, whole_heads;
@@ -59,14 +62,23 @@ static const PlanRow kPlanTable[] = {
 constexpr int kTableCus = 256;  // the table was measured on a 256-CU device
 
 // Applies a table row to the actual t: the split factor is kept, the pieces are re-cut.
-static bool plan_from_table(int precision, int bh, int Dh, int t, float p, int cus, ffa_launch_plan* plan) {
-    if (cus != kTableCus) return false;
+// Returns kNoRow when no row covers the problem, kRowKeepsRules when one does and records that the
+// rules' plan was within 3 % of the best (the grid is not consulted then either), kRowOverrides
+// when *plan now holds the row's plan.
+enum { kNoRow = 0, kRowKeepsRules = 1, kRowOverrides = 2 };
+static int plan_from_table(int precision, int bh, int Dh, int t, float p, int cus, ffa_launch_plan* plan) {
+    if (cus != kTableCus) return kNoRow;
     const int pruned = p > 0.f ? 1 : 0;
     const int ntiles = num_tiles(t);
-    for (const PlanRow* r = kPlanTable; r->precision != 0; ++r) {
-        if (!r->override_rules) continue;  // a record of the sweep: the rules' plan was kept
-        if (r->precision != precision || r->head_dim != Dh || r->pairs != bh || r->pruned != pruned) continue;
-        if (t < r->t_lo || t > r->t_hi) continue;
+    // Rows of different sweeps may overlap in t: the one whose centre is nearest decides.
+    const PlanRow* r = nullptr;
+    for (const PlanRow* c = kPlanTable; c->precision != 0; ++c) {
+        if (c->precision != precision || c->head_dim != Dh || c->pairs != bh || c->pruned != pruned) continue;
+        if (t < c->t_lo || t > c->t_hi) continue;
+        if (r == nullptr || abs(2 * t - c->t_lo - c->t_hi) < abs(2 * t - r->t_lo - r->t_hi)) r = c;
+    }
+    if (r != nullptr) {
+        if (!r->override_rules) return kRowKeepsRules;
         int n_splits = r->n_splits < 1 ? 1 : r->n_splits;
         if (n_splits > ntiles) n_splits = ntiles;
         const int tps = ceil_div(ntiles, n_splits);
@@ -75,13 +87,93 @@ static bool plan_from_table(int precision, int bh, int Dh, int t, float p, int c
         plan->threads_per_key = r->tpk;
         plan->keys_per_wave = kTileKeys / r->tpk;
         plan->whole_heads = r->kind == FFA_LAUNCH_SPLIT ? (n_splits == 1 ? bh : r->whole_heads) : 0;
-        return validate_plan(*plan, precision, Dh, bh, t, p) == FFA_OK;
+        return validate_plan(*plan, precision, Dh, bh, t, p) == FFA_OK ? kRowOverrides : kRowKeepsRules;
     }
-    return false;
+    return kNoRow;
+}
+
+// ---------------------------------------------------------------------------------------
+// The grid (ffa_plan_grid.inc, written by `python bench.py --sweep-plans grid`): the same sweep
+// over a grid of pairs x head dimension x length x pruned-or-not, for problems away from the
+// table's shapes.  A problem takes the nearest row of its (precision, head dimension, pruned)
+// class, if one lies within a factor of sqrt 2 in both the number of pairs and the length; where
+// that row overrides the rules, its launch kind, wave count and lanes per key are kept and its
+// workgroup count is re-cut for the problem at hand.
+struct GridRow {
+    int override_rules, precision, head_dim, pairs, t, pruned;
+    int kind, waves, tpk, n_splits, whole_heads;
+    float chosen_us, best_us, rule_us;
+};
+static const GridRow kPlanGrid[] = {
+#define FFA_GRID_ROW(ov, prec, dh, pairs, t, pruned, kind, waves, tpk, ns, whole, chosen, best, rule) \
+    {ov, prec, dh, pairs, t, pruned, kind, waves, tpk, ns, whole, chosen, best, rule},
+#include "ffa_plan_grid.inc"
+#undef FFA_GRID_ROW
+    {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0.f, 0.f, 0.f}  // sentinel
+};
+
+static const GridRow* nearest_grid_row(int precision, int bh, int Dh, int t, int pruned) {
+    const GridRow* best = nullptr;
+    double best_d = 1e30;
+    for (const GridRow* r = kPlanGrid; r->precision != 0; ++r) {
+        if (r->precision != precision || r->head_dim != Dh || r->pruned != pruned) continue;
+        const double dp = fabs(log2((double)bh / r->pairs)), dt = fabs(log2((t + 1.0) / (r->t + 1.0)));
+        if (dp > 0.5 || dt > 0.5) continue;
+        if (dp + dt < best_d) {
+            best_d = dp + dt;
+            best = r;
+        }
+    }
+    return best;
+}
+
+static bool plan_from_grid(int precision, int bh, int Dh, int t, float p, int cus, ffa_launch_plan* plan) {
+    if (cus != kTableCus) return false;
+    const GridRow* r = nearest_grid_row(precision, bh, Dh, t, p > 0.f ? 1 : 0);
+    if (r == nullptr || !r->override_rules) return false;
+    const int ntiles = num_tiles(t);
+    int whole = 0;
+    double n = 1.0;
+    if (r->kind == FFA_LAUNCH_TWO_PASS) {
+        n = (double)r->n_splits * r->pairs / bh;
+    } else if (r->kind == FFA_LAUNCH_SPLIT) {
+        if (r->n_splits <= 1 || r->whole_heads >= r->pairs) {
+            whole = bh;  // one workgroup per pair
+        } else if (r->whole_heads > 0) {
+            // Hybrid: whole pairs in multiples of the CU count, the row's piece count for the rest.
+            whole = (bh / cus) * cus;
+            const int rest = bh - whole;
+            if (rest == 0) whole = bh;
+            else n = (double)r->n_splits * (r->pairs - r->whole_heads) / rest;
+        } else {
+            n = (double)r->n_splits * r->pairs / bh;
+        }
+    }
+    int n_splits = (int)(n + 0.5);
+    const int cap = max_splits_for(bh - (whole < bh ? whole : 0), t + 1);
+    if (n_splits > cap) n_splits = cap;
+    if (n_splits > ntiles) n_splits = ntiles;
+    if (n_splits < 1) n_splits = 1;
+    const int tps = ceil_div(ntiles, n_splits);
+    n_splits = ceil_div(ntiles, tps);
+    fill(plan, r->kind, r->waves, n_splits, tps);
+    plan->threads_per_key = r->tpk;
+    plan->keys_per_wave = kTileKeys / r->tpk;
+    if (r->kind == FFA_LAUNCH_SPLIT) plan->whole_heads = n_splits == 1 ? bh : whole;
+    return validate_plan(*plan, precision, Dh, bh, t, p) == FFA_OK;
 }
 
 static int plan_by_rules(int precision, int B, int H, int Dh, int t, float p, int use_default, int cus,
                          ffa_launch_plan* plan);
+
+int plan_source(int precision, int B, int H, int Dh, int t, float p, int cus) {
+    ffa_launch_plan tmp;
+    if (cus <= 0) cus = 256;
+    const int row = plan_from_table(precision, B * H, Dh, t, p, cus, &tmp);
+    if (row == kRowOverrides) return 1;
+    if (row == kNoRow && plan_from_grid(precision, B * H, Dh, t, p, cus, &tmp)) return 2;
+    return 0;
+}
 
 int plan_launch(int precision, int B, int H, int Dh, int t, float p, int use_default, int cus,
                 ffa_launch_plan* plan) {
@@ -93,7 +185,9 @@ int plan_launch_ex(int precision, int B, int H, int Dh, int t, float p, int use_
     const int st = plan_by_rules(precision, B, H, Dh, t, p, use_default, cus, plan);
     if (st != FFA_OK || use_default || !use_table) return st;
     ffa_launch_plan from_table;
-    if (plan_from_table(precision, B * H, Dh, t, p, cus <= 0 ? 256 : cus, &from_table)) *plan = from_table;
+    const int row = plan_from_table(precision, B * H, Dh, t, p, cus <= 0 ? 256 : cus, &from_table);
+    if (row == kRowOverrides) *plan = from_table;
+    else if (row == kNoRow && plan_from_grid(precision, B * H, Dh, t, p, cus <= 0 ? 256 : cus, &from_table)) *plan = from_table;
     return FFA_OK;
 }
 
@@ -122,56 +216,67 @@ static int plan_by_rules(int precision, int B, int H, int Dh, int t, float p, in
     }
 
     if (p > 0.f) {
-        // Pruning needs the global max and sum before it may touch V.  With at least half a
-        // pair per CU and scores that fit LDS: one workgroup per (b,h), as many waves as
-        // there are tiles to keep in flight (up to 16).  Otherwise the two-pass pair of
-        // kernels, cut along the sequence.
-        if (fits_wg && 2 * bh >= cus) {
-            fill(plan, FFA_LAUNCH_WORKGROUP, wg_waves_for(ntiles, ceil_div(ntiles, 4)), 1, ntiles);
-            return FFA_OK;
-        }
-        // Measured on MI355X (8192 keys, 32 and 128 pairs): both kernels of the pair carry
-        // only half of a tile's loads each, so they want twice the workgroups of the exact
-        // path -- about two 8-wave workgroups per CU -- as long as every wave keeps a tile.
-        int n_splits = 2 * cus / bh;
+        // Pruning needs the global max and sum before it may touch V: either one workgroup per
+        // (b,h) with the scores in LDS, or the two-pass pair of kernels cut along the sequence.
+        // The second launch and the merge of the pieces cost about a dozen tile-times (of any
+        // width), and a cut in two or three gains little, so cutting a pair into n pieces pays
+        // from ntiles (1 - 1.7/n) >= 12 on, and never with a pair or more per CU (grid sweep: 16
+        // and 32 pairs go two-pass from 1024 keys, 64 pairs from 2048, 128 pairs from 8192; at 256
+        // pairs and more the one-workgroup kernel wins at every length).
+        // Both kernels of the pair carry only half of a tile's loads each, so from 4096 keys on
+        // they want twice the workgroups of the exact path -- about two 8-wave workgroups per CU;
+        // below that one workgroup per CU (grid sweep: 32 pairs x 1024 keys 8.4 vs 9.1 us).
+        int n_splits = (ntiles >= 64 ? 2 : 1) * cus / bh;
         if (n_splits > ntiles) n_splits = ntiles;
         const int cap = max_splits_for(bh, t + 1);
         if (n_splits > cap) n_splits = cap;
         if (n_splits < 1) n_splits = 1;
+        const bool cut_pays = bh < cus && n_splits > 1 && ntiles * (n_splits - 1.7) >= 12.0 * n_splits;
+        if (fits_wg && !cut_pays) {
+            // Waves: one tile or two per wave up to 8 waves; 16 waves only for very long sequences
+            // with a whole number of pairs per CU (512 pairs x 8192 keys); 4 waves when some CUs get
+            // a second workgroup (320 pairs: 5-9 % at every length).
+            int want = ntiles <= 5 ? 4 : 8;
+            if (bh % cus == 0 && ntiles >= 128) want = 16;
+            if (bh > cus && bh % cus != 0) want = 4;
+            fill(plan, FFA_LAUNCH_WORKGROUP, wg_waves_for(ntiles, want), 1, ntiles);
+            return FFA_OK;
+        }
         const int tps = ceil_div(ntiles, n_splits);
         n_splits = ceil_div(ntiles, tps);
-        const int waves = wg_waves_for(tps, 8);
-        if (n_splits == 1 && fits_wg)  // nothing to cut: the single kernel does the same work
-            fill(plan, FFA_LAUNCH_WORKGROUP, wg_waves_for(ntiles, ceil_div(ntiles, 4)), 1, ntiles);
-        else
-            fill(plan, FFA_LAUNCH_TWO_PASS, waves, n_splits, tps);
+        fill(plan, FFA_LAUNCH_TWO_PASS, tps <= 4 ? 4 : 8, n_splits, tps);
         return FFA_OK;
     }
 
     // Exact path.  Measured on MI355X: the launch runs best with about one 4-wave workgroup
     // per CU, each walking a long run of tiles, and with as few cross-workgroup merges as
-    // possible at the END of the kernel (a merge is a chain of three HBM-latency hops).
+    // possible at the END of the kernel (a merge is a chain of three memory round trips).
     //  - At least one (batch, head) pair per CU: whole pairs go to single workgroups in
     //    multiples of the CU count (every CU gets the same number, LDS-only merge); only the
     //    remainder is split, into ceil(CUs/rest) pieces per pair, so that the pieces also
     //    cover all CUs and are done, merges included, long before the whole pairs are.
     //  - Fewer pairs than CUs: floor(CUs/pairs) pieces per pair (one workgroup per CU), but
-    //    never so many that a wave is left without a tile.
-    //  - Long sequences with at least one pair per CU: the one-workgroup kernel with 16 waves
-    //    (separate K and V phases).  Every exact launch is within 1 % of the others there
-    //    (512 pairs x 8192 keys: 163 to 166 us for the split kernel with 4 or 8 waves and this
-    //    kernel with 4, 8 or 16 waves); this one also serves the pruned steps of such shapes.
-    //    Below 4096 keys the split kernel is ahead.
-    if (bh >= cus && ntiles >= 64 && fits_wg) {
+    //    never so many that a wave is left without a tile -- and only where the split saves more
+    //    than its merge costs.  The merge chain is worth the time of about ten 16 KiB tiles, so a
+    //    cut into n pieces pays from ntiles (tile bytes / 16 KiB) (1 - 1/n) >= 10 on (grid sweep:
+    //    at Dh = 64 fp16 128 pairs stay whole up to 1024 keys, 16 pairs up to 256); below that
+    //    every pair is one workgroup of up to 8 waves.
+    //  - Long sequences with a whole number of pairs per CU: the one-workgroup kernel with 16
+    //    waves (separate K and V phases; 512 pairs x 8192 keys: all exact launches within 1 %).
+    //    With a remainder the hybrid launch is 15-20 % ahead (320 pairs from 4096 keys on).
+    //  - Wide rows (16 or more 16-byte chunks per key: Dh 128 / 256 in fp16, Dh 64 / 128 in fp32):
+    //    four lanes per key, so that a tile's loads are all in flight at once (grid sweep: 5-25 %
+    //    at every length below two pairs per CU), with 8 waves per workgroup below one pair per CU.
+    int whole = (bh / cus) * cus;
+    const int rest = bh - whole;
+    if (rest == 0 && ntiles >= 64 && fits_wg) {
         fill(plan, FFA_LAUNCH_WORKGROUP, 16, 1, ntiles);
         return FFA_OK;
     }
     const int waves = wg_waves_for(ntiles, 4);
-    int whole = (bh / cus) * cus;
-    const int rest = bh - whole;
     int n_splits = 1;
     if (whole > 0) {
-        if (rest > 0) n_splits = ceil_div(cus, rest);
+        if (rest > 0 && ntiles >= 8) n_splits = ceil_div(cus, rest);
     } else {
         n_splits = cus / bh;
     }
@@ -179,18 +284,24 @@ static int plan_by_rules(int precision, int B, int H, int Dh, int t, float p, in
     const int cap = max_splits_for(rest > 0 ? rest : bh, t + 1);
     if (n_splits > cap) n_splits = cap;
     if (n_splits < 1) n_splits = 1;
+    const int nch = Dh * (precision / 8) / 16;  // 16-byte chunks per key: a 64-key tile is nch x 2 KiB
+    if (whole == 0 && n_splits > 1 && (long long)ntiles * nch * (n_splits - 1) < 80ll * n_splits) n_splits = 1;
     const int tps = ceil_div(ntiles, n_splits);
     n_splits = ceil_div(ntiles, tps);
-    if (n_splits == 1) whole = bh;  // nothing left to split: plain one-workgroup-per-pair
-    // Between CUs/2 and CUs pairs nothing can be cut without doubling up CUs; the idle CUs
-    // are made up for with 8 waves per workgroup (160 pairs, 1000 keys: 9.3 vs 9.8 us).
-    if (n_splits == 1 && bh < cus) {
-        fill(plan, FFA_LAUNCH_SPLIT, wg_waves_for(ntiles, 8), 1, ntiles);
+    const int tpk = (nch >= 16 && bh < 2 * cus && tpk_supported(precision, Dh, 4)) ? 4 : 1;
+    if (n_splits == 1) {
+        // Nothing is cut: one workgroup per pair.  Below one pair per CU the idle CUs are made up
+        // for with 8 waves per workgroup (160 pairs, 1000 keys: 9.3 vs 9.8 us).
+        const int w = bh < cus ? wg_waves_for(ntiles * tpk, 8) : waves;
+        fill(plan, FFA_LAUNCH_SPLIT, tpk > 1 && w < 4 ? 4 : w, 1, ntiles);
         plan->whole_heads = bh;
-        return FFA_OK;
+    } else {
+        const int w = tpk > 1 ? (bh < cus ? 8 : 4) : waves;
+        fill(plan, FFA_LAUNCH_SPLIT, w, n_splits, tps);
+        plan->whole_heads = whole;
     }
-    fill(plan, FFA_LAUNCH_SPLIT, waves, n_splits, tps);
-    plan->whole_heads = whole;
+    plan->threads_per_key = tpk;
+    plan->keys_per_wave = kTileKeys / tpk;
     return FFA_OK;
 }
 

@@ -124,6 +124,13 @@ int ffa_plan_launch_rules(int precision, int batch_size, int head_num, int head_
                           int t, float prob_thresh, int use_default_kernel_launch,
                           int compute_units, ffa_launch_plan* plan);
 
+/* Where ffa_plan_launch takes the tuned plan of a problem from: 0 = the rules, 1 = a row of the
+ * table measured at the BASELINE shapes (exact match), 2 = the nearest row of the measured grid
+ * (csrc/ffa_plan_grid.inc, `python bench.py --sweep-plans grid`).  Negative = bad arguments.  No
+ * counterpart in the reference, whose fitted model (kernel_launch_utils.h:85-132) has one source. */
+int ffa_plan_source(int precision, int batch_size, int head_num, int head_dim, int t,
+                    float prob_thresh, int compute_units);
+
 /* Bytes of device workspace sufficient for ANY plan this library produces for the
  * given problem (arrival counters, split partials, two-pass scores). */
 size_t ffa_workspace_bytes(int batch_size, int head_num, int head_dim, int max_seq_len);

@@ -138,23 +138,24 @@ def test_opt13b_shape_b2_last_step():
 @pytest.mark.parametrize("t0", [2000, 2060, 2250])
 def test_gptj_shape_steps(t0):
     """BASELINE configs[3]: B=8, 16 heads x 256, fp16, prompt 2000, max_len 2256.  Steps around
-    t0 with the launch the library plans (one lane per key below 2065 keys, four lanes per key
-    from there on: the planner's measured table) and the default launch, against the oracle;
-    caches bit for bit."""
+    t0 with the launch the library plans (four lanes per key: wide rows), the same split with one
+    lane per key, and the default launch, against the oracle; caches bit for bit."""
     B, H, Dh, prec, Lmax, steps = 8, 16, 256, 16, 2256, 6
     rng, K, V = rand_inputs(500 + t0, B, H, t0, Dh, prec, kv_scale=0.5)
     scale = 1.0 / 16.0
     kinds = set()
-    for use_default in (False, True):
+    for launch in ("library", "one lane per key", "default"):
         sess = CApiSession(K, V, Lmax)
         kc, vc = O.pack_k_cache(K, Lmax), O.pack_v_cache(V, Lmax)
         worst = 0.0
         for i in range(steps):
             t = t0 + i
             q, k, v = rand_token(rng, B, H, Dh, prec)
-            plan = capi.plan_launch(prec, B, H, Dh, t, 0.0, use_default)
+            plan = capi.plan_launch(prec, B, H, Dh, t, 0.0, launch == "default")
+            if launch == "one lane per key":
+                plan = capi.make_plan(capi.FFA_LAUNCH_SPLIT, 4, plan.n_splits, plan.tiles_per_split, 0, plan.whole_heads)
             kinds.add((plan.kind, plan.threads_per_key))
-            _say("gptj", use_default, t, plan)
+            _say("gptj", launch, t, plan)
             got = sess.step(q, k, v, scale, t, plan=plan)
             want = O.decode_step(q, k, v, kc, vc, scale, t, acc=np.float64)
             worst = max(worst, float(np.abs(got - want).max()))
@@ -163,8 +164,7 @@ def test_gptj_shape_steps(t0):
         n = t0 + steps                       # slots beyond are untouched (and unspecified) on both sides
         np.testing.assert_array_equal(gk[:, :, :, :n].view(np.uint16), kc[:, :, :, :n].view(np.uint16))
         np.testing.assert_array_equal(gv[:, :, :n].view(np.uint16), vc[:, :, :n].view(np.uint16))
-    if t0 == 2060:      # the steps cross from one lane per key to four
-        assert (capi.FFA_LAUNCH_SPLIT, 1) in kinds and (capi.FFA_LAUNCH_SPLIT, 4) in kinds
+    assert kinds == {(capi.FFA_LAUNCH_SPLIT, 4), (capi.FFA_LAUNCH_SPLIT, 1), (capi.FFA_LAUNCH_WORKGROUP, 1)}, kinds
 
 
 # ------------------------------------------------------------------ configs[4]: pruned sweep, B = 16

@@ -258,9 +258,9 @@ def test_hook_with_hip_engine(family, dtype, tol):
 
 
 def small_gptj(dtype=torch.float32):
-    """Four heads of 64, room for 256 positions: long enough for the launch plan of a decode to
+    """Four heads of 64, room for 1024 positions: long enough for the launch plan of a decode to
     move from one workgroup per head to sequence-split launches."""
-    cfg = transformers.GPTJConfig(vocab_size=96, n_positions=256, n_embd=256, n_layer=2, n_head=4, rotary_dim=32,
+    cfg = transformers.GPTJConfig(vocab_size=96, n_positions=1024, n_embd=256, n_layer=2, n_head=4, rotary_dim=32,
                                   n_inner=256, resid_pdrop=0.0, embd_pdrop=0.0, attn_pdrop=0.0,
                                   bos_token_id=2, eos_token_id=2)
     torch.manual_seed(0)
@@ -270,12 +270,18 @@ def small_gptj(dtype=torch.float32):
 @pytest.mark.gpu
 @pytest.mark.parametrize("dtype,tol", [(torch.float32, 2e-4), (torch.float16, 3e-2)])
 def test_long_decode_with_fused_rotary_crosses_launch_plans(dtype, tol):
-    """170 decode steps from a 9-token prompt through the hook with the rotary embedding inside the
-    engine's call, one engine (one workspace) per layer for the whole decode; the logits of every
-    step against transformers' own cache.  The engine's plan changes kind on the way."""
+    """170 decode steps from a long prompt (one sample left-padded by 37) through the hook with
+    the rotary embedding inside the engine's call, one engine (one workspace) per layer for the
+    whole decode; the logits of every step against transformers' own cache.  The engine's plan
+    changes from one workgroup per head to sequence-split launches on the way."""
     print("hf long decode", dtype, flush=True)
     model = small_gptj(dtype).to("cuda:0")
-    ids, mask = padded_batch("cuda:0")
+    g = torch.Generator().manual_seed(5)
+    prompt, pad = (740 if dtype == torch.float16 else 430), 37    # the plans switch at 832 / 512 cached keys
+    ids = torch.randint(3, 96, (2, prompt), generator=g).to("cuda:0")
+    mask = torch.ones_like(ids)
+    ids[1, :pad] = 1
+    mask[1, :pad] = 0
     steps = 170
     want, _ = teacher_forced_logits(model, ids, mask, steps, None)
     hf.enable(model, fused_rotary=True)
@@ -285,5 +291,5 @@ def test_long_decode_with_fused_rotary_crosses_launch_plans(dtype, tol):
     err = (got - want).abs().amax(dim=(1, 2))
     assert float(err.max()) < tol, (int(err.argmax()), float(err.max()))
     engine = cache.layers[0].engine
-    split = {engine.launch_plan(t, 0.0)[4] > 1 for t in range(9, 9 + steps)}
+    split = {engine.launch_plan(t, 0.0)[4] > 1 for t in range(prompt, prompt + steps)}
     assert split == {False, True}, "the decode never crossed from unsplit to sequence-split launches"
