@@ -158,6 +158,25 @@ class Workload:
         if rc != 0:
             raise RuntimeError(f"ffa_attention failed: {self.capi.status_string(rc)}")
 
+    def floor_plan(self, t):
+        """The step's plan as the load-floor probe takes it (split launch, one lane per key, 2 / 4 / 8
+        waves: the same grid and bytes), or None when the step is not a split launch."""
+        p = self.plan_for(t)
+        if p.kind != self.capi.FFA_LAUNCH_SPLIT:
+            return None
+        waves = min((2, 4, 8), key=lambda w: abs(w - p.waves_per_wg))
+        return self.capi.make_plan(p.kind, waves, p.n_splits, p.tiles_per_split, 0, p.whole_heads)
+
+    def launch_floor(self, i, stream_ptr):
+        """The load floor of step i: same grid, same loads, nothing else (ffa_load_floor)."""
+        t = self.t_of(i)
+        l = i % self.layers
+        rc = self.lib.ffa_load_floor(self.precision, self.B, self.H, self.Dh, self.Lmax, t, self.kc[l].data_ptr(),
+                                     self.vc[l].data_ptr(), None, 1, C.byref(self.floor_plan(t)),
+                                     self.out.data_ptr(), stream_ptr)
+        if rc != 0:
+            raise RuntimeError(f"ffa_load_floor failed: {self.capi.status_string(rc)}")
+
     def mean_bytes(self, launches=None):
         n = launches or self.steps
         return sum(algorithmic_bytes(self.B, self.H, self.Dh, self.t_of(i), self.elem) for i in range(n)) / n
@@ -195,9 +214,13 @@ def launches_for(wl, steps, warmup):
     return steps * passes
 
 
-def run_graph(wl, launches, replays=5):
-    """Returns the per-replay times (ms) of a graph holding `launches` launches."""
+def run_graph(wl, launches, replays=5, floor=False):
+    """Returns the per-replay times (ms) of a graph holding `launches` launches (floor: of the
+    load-floor probe of each step instead of the step itself)."""
     torch = wl.torch
+    if floor:
+        import types
+        wl = types.SimpleNamespace(torch=torch, layers=wl.layers, launch=wl.launch_floor)
     side = torch.cuda.Stream()
     side.wait_stream(torch.cuda.current_stream())
     with torch.cuda.stream(side):          # warm-up on the capture stream, eager
@@ -636,6 +659,12 @@ def measure_row(name, use_default=False, steps=32, eager=True):
            "plan": repr(wl.plan_for(wl.t_of(0)))}
     if eager:
         row["eager_capi_us_per_step"] = round(run_capi(wl, n) * 1e3 / n, 2)
+    if not use_default and all(wl.floor_plan(wl.t_of(i)) is not None for i in range(steps)):
+        # The same launches with every load and nothing else: what this launch shape could reach
+        # with free arithmetic and free merges.
+        fl = median(run_graph(wl, n, floor=True)) * 1e3 / n
+        row["load_floor_us_per_step"] = round(fl, 2)
+        row["of_load_floor"] = round(fl / us, 3)
     del wl
     torch.cuda.empty_cache()
     return row
@@ -1051,10 +1080,13 @@ def main():
     launches = launches_for(wl, steps, warmup)
 
     res, replays_us = {}, None
+    floor_us = None
     if "graph" in legs:
         reps = run_graph(wl, launches)
         replays_us = [round(ms * 1e3 / launches, 3) for ms in reps]
         res["graph"] = median(reps)
+        if all(wl.floor_plan(wl.t_of(i)) is not None for i in range(steps)):
+            floor_us = median(run_graph(wl, launches, floor=True)) * 1e3 / launches
     if "capi" in legs:
         res["capi"] = run_capi(wl, launches)
     if "ext" in legs:
@@ -1087,6 +1119,11 @@ def main():
                      "kernel": {0: "ffa_decode_wg_kernel", 1: "ffa_decode_split_kernel"}.get(plan0.kind, "two-pass pair"),
                      "launch_us": round(us_step, 3)},
     }
+    if floor_us is not None:
+        # the same launches with every load and nothing else (ffa_load_floor): what this launch
+        # shape could reach with free arithmetic and free merges
+        out["roofline"]["load_floor_us"] = round(floor_us, 3)
+        out["roofline"]["of_load_floor"] = round(floor_us / us_step, 4)
     if replays_us is not None:
         out["graph_replays_us_per_step"] = replays_us
     for leg in ("capi", "ext"):

@@ -86,6 +86,7 @@ SIGNATURES = {
                               _BI_P, _vp, _sz, _vp]),
     "ffa_attention_static_scratch": (_i, [_i, _i, _i, _i, _i, _f, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _f,
                                           _PLAN_P, _i, _TT_P, _BI_P, _vp]),
+    "ffa_load_floor": (_i, [_i, _i, _i, _i, _i, _i, _vp, _vp, _vp, _i, _PLAN_P, _vp, _vp]),
 }
 
 _lib = None

@@ -247,6 +247,33 @@ int ffa_attention_ex(int precision, int batch_size, int head_num, int head_dim, 
     return run_decode(a, plan, workspace, workspace_bytes);
 }
 
+int ffa_load_floor(int precision, int batch_size, int head_num, int head_dim, int max_seq_len, int t,
+                   const void* k_cache, const void* v_cache, const int* seq_lengths, int right_or_no_padding,
+                   const ffa_launch_plan* plan, void* sink, void* stream) {
+    if (plan == nullptr || sink == nullptr) return FFA_ERR_NULL_POINTER;
+    if (plan->kind != FFA_LAUNCH_SPLIT || plan->threads_per_key != 1 ||
+        (plan->waves_per_wg != 2 && plan->waves_per_wg != 4 && plan->waves_per_wg != 8))
+        return FFA_ERR_PLAN;
+    DecodeArgs a;
+    a.precision = precision;
+    a.B = batch_size; a.H = head_num; a.Dh = head_dim; a.Lmax = max_seq_len; a.t = t;
+    a.scale = 1.f; a.p = 0.f;
+    // The probe reads the caches only; q, k, v stand in as non-null, aligned addresses that it never touches.
+    a.q = a.k = a.v = sink;
+    a.k_cache = const_cast<void*>(k_cache); a.v_cache = const_cast<void*>(v_cache); a.out = sink;
+    a.seq_lengths = seq_lengths;
+    a.right_or_no_padding = right_or_no_padding;
+    a.kept_count = nullptr; a.skip_mask = nullptr;
+    a.stream = stream;
+    a.floor_probe = true;
+    int st = validate_decode(a);
+    if (st != FFA_OK) return st;
+    st = validate_plan(*plan, planner_precision(precision), head_dim, batch_size * head_num, t, 0.f);
+    if (st != FFA_OK) return st;
+    const WorkspaceView none = {nullptr, nullptr, nullptr, nullptr, 0};
+    return launch_decode(a, *plan, none);
+}
+
 int ffa_attention_static_scratch(int precision, int batch_size, int head_num, int head_dim,
                                   int max_seq_len, float softmax_scale, int t, const void* q,
                                   const void* k, const void* v, void* k_cache, void* v_cache,

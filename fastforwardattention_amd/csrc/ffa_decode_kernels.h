@@ -1051,6 +1051,71 @@ ffa_decode_split_tpk_kernel(HOT_PARAMS_DECL, const DecodeParams P_rest) {
     if (has_token) token_store<T, DH>(tok, kc_bh, vc_bh, tlen, P.Lmax, lane);
 }
 
+// ---------------------------------------------------------------------------------------
+// Load floor of a split launch (ffa_load_floor): the grid, the workgroups, the piece mapping, the
+// tile order and the addresses of ffa_decode_split_kernel, every 16-byte load of every tile issued
+// the same way (at most 16 in flight per wave) -- and nothing else: no arithmetic on the data, no
+// merge, no output.  What it takes is what the memory system gives this launch shape; the decode
+// kernel's distance from it is the cost of its arithmetic and of its merges.  The loaded words
+// are folded with XOR so that the loads cannot be dropped; the fold is stored only if it equals a
+// value it never takes.
+template <typename T, int DH, int NW>
+__global__ void __launch_bounds__((NW + 1) * 64) ffa_load_floor_kernel(HOT_PARAMS_DECL, const DecodeParams P_rest) {
+    const DecodeParams P = with_hot_params(P_rest, HOT_PARAMS_USE);
+    using G = Geo<T, DH>;
+    constexpr int NCH = G::NCH, LPR = G::LPR, RPI = G::RPI, NVL = G::NVL;
+    constexpr int GRP = 8;  // loads per group: one group of K and one of V in flight, as in the decode kernel
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const PieceOf piece(P, (int)blockIdx.x);
+    const int bh = piece.bh, split = piece.split, n_splits = piece.n_splits;
+    int tlen, first;
+    step_bounds(P, P.seq_lengths != nullptr ? bh / P.H : 0, tlen, first);
+    if (wave == NW || tlen <= 0) return;  // the token wave loads nothing from the caches
+    const size_t head_bytes = (size_t)P.Lmax * DH * sizeof(T);
+    const char* kc_bh = reinterpret_cast<const char*>(P.k_cache) + (size_t)bh * head_bytes;
+    const char* vc_bh = reinterpret_cast<const char*>(P.v_cache) + (size_t)bh * head_bytes;
+    const int ntiles = (tlen + kWave - 1) / kWave;
+    const int tps = n_splits == 1 ? ntiles : P.tiles_per_split;
+    const int tile_lo = max(split * tps, first / kWave);
+    const int tile_hi = min(ntiles, (split + 1) * tps);
+    const int last_key = tlen - 1;
+    const int rg = lane / LPR, dch = min(lane % LPR, NCH - 1);
+    const size_t kstr = (size_t)P.Lmax * 16;
+    const TileOrder order(tile_lo, tile_hi, (unsigned)(bh * n_splits + split));
+    uint4 fold = make_uint4(0u, 0u, 0u, 0u);
+    auto take = [&](const uint4& v) { fold.x ^= v.x; fold.y ^= v.y; fold.z ^= v.z; fold.w ^= v.w; };
+    for (int idx = wave; idx < order.n; idx += NW) {
+        const int tile = order.at(idx);
+        const char* kp = kc_bh + (size_t)min(tile * kWave + lane, last_key) * 16;
+        constexpr int NG = ((NCH > NVL ? NCH : NVL) + GRP - 1) / GRP;
+#pragma unroll
+        for (int g = 0; g < NG; ++g) {
+            uint4 kv[GRP], vv[GRP];
+#pragma unroll
+            for (int c = 0; c < GRP; ++c) {
+                kv[c] = make_uint4(0u, 0u, 0u, 0u);
+                if (g * GRP + c < NCH) kv[c] = ld16(kp + (size_t)(g * GRP + c) * kstr);
+            }
+#pragma unroll
+            for (int j = 0; j < GRP; ++j) {
+                vv[j] = make_uint4(0u, 0u, 0u, 0u);
+                if (g * GRP + j < NVL) {
+                    const int row = min(tile * kWave + (g * GRP + j) * RPI + rg, last_key);
+                    vv[j] = ld16(vc_bh + ((size_t)row * NCH + dch) * 16);
+                }
+            }
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int c = 0; c < GRP; ++c) take(kv[c]);
+#pragma unroll
+            for (int j = 0; j < GRP; ++j) take(vv[j]);
+        }
+    }
+    if (fold.x == 0x9e3779b9u && fold.y == 0x7f4a7c15u && fold.z == 0xf39cc060u && fold.w == 0x5cedc834u)
+        *reinterpret_cast<uint4*>(P.out) = fold;
+}
+
 // Merge kernel of FFA_COMBINE_KERNEL: one wave per split (b,h) pair, log-sum-exp over its
 // partials.
 template <typename T, int DH>
@@ -1598,8 +1663,29 @@ static int launch_wg(const DecodeParams& P, size_t lds_bytes, hipStream_t st) {
     return check_launch();
 }
 
+template <typename T, int DH, int NW>
+static int launch_floor(const DecodeParams& P, hipStream_t st) {
+    const int n_split_heads = P.bh_total - P.n_whole;
+    const dim3 grid((unsigned)(P.n_whole + n_split_heads * P.n_splits));
+    hipLaunchKernelGGL((ffa_load_floor_kernel<T, DH, NW>), grid, dim3((NW + 1) * 64), 0, st, HOT_PARAMS_OF(P), P);
+    return check_launch();
+}
+
 template <typename T, int DH, bool BEAM, bool XFORM>
 static int dispatch_waves(const DecodeParams& P, const ffa_launch_plan& plan, hipStream_t st) {
+    if (P.floor_probe) {
+        if constexpr (!BEAM && !XFORM) {
+            if (plan.kind != FFA_LAUNCH_SPLIT || plan.threads_per_key != 1) return FFA_ERR_PLAN;
+            switch (plan.waves_per_wg) {
+                case 2: return launch_floor<T, DH, 2>(P, st);
+                case 4: return launch_floor<T, DH, 4>(P, st);
+                case 8: return launch_floor<T, DH, 8>(P, st);
+                default: return FFA_ERR_PLAN;
+            }
+        } else {
+            return FFA_ERR_PLAN;
+        }
+    }
     if (plan.kind == FFA_LAUNCH_SPLIT && plan.threads_per_key > 1) {
         if constexpr (DH == 80) {  // 10 / 20 chunks per key do not divide among 2 or 4 lanes
             return FFA_ERR_PLAN;

@@ -42,6 +42,9 @@ struct DecodeArgs {
     const int* cache_indir = nullptr;
     int beam_width = 1;
 
+    // ffa_load_floor: launch the load-only probe of the plan instead of the decode kernel.
+    bool floor_probe = false;
+
     bool transforms_token() const { return q_bias || k_bias || v_bias || rotary_dim > 0; }
 };
 
@@ -78,6 +81,7 @@ struct DecodeParams {
     int rotary_dim;          // 0 = none
     int xform;               // any bias or a rotary embedding present
     double rotary_coef;      // -2 log2(base) / rotary_dim: angle of pair z = pos * 2^(z * coef)
+    int floor_probe;         // launch ffa_load_floor_kernel instead of the decode kernel
 };
 
 // Carved-up workspace for a given plan.

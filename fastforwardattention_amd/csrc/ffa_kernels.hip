@@ -131,6 +131,7 @@ int launch_decode(const DecodeArgs& a, const ffa_launch_plan& plan, const Worksp
     P.q_bias = a.q_bias; P.k_bias = a.k_bias; P.v_bias = a.v_bias;
     P.rotary_dim = a.rotary_dim;
     P.xform = a.transforms_token() ? 1 : 0;
+    P.floor_probe = a.floor_probe ? 1 : 0;
     P.rotary_coef = a.rotary_dim > 0 ? -2.0 * log2((double)a.rotary_base) / (double)a.rotary_dim : 0.0;
     // The transform is a compile-time switch of the kernels: the plain step carries none of its code.
     if (P.xform) {

@@ -277,6 +277,19 @@ int ffa_attention_static_scratch(int precision, int batch_size, int head_num, in
                                   const ffa_token_transform* transform,
                                   const ffa_beam_indirection* beams, void* stream);
 
+/*
+ * Measurement aid, no counterpart in the reference: the load floor of an FFA_LAUNCH_SPLIT plan
+ * with one lane per key and 2, 4 or 8 waves.  Launches the grid, the workgroups and the tile walk
+ * of the decode kernel for this plan and issues every 16-byte load of K and V that the step would
+ * issue (cached keys 0 .. t-1), the same number in flight per wave -- no arithmetic, no merge, no
+ * output.  Its duration is what the memory system gives this launch shape; bench.py reports the
+ * decode kernels against it.  `sink`: 16 bytes of device memory, 16-byte aligned (the probe stores
+ * to it only if the XOR of everything it loaded equals one fixed value); the caches are only read.
+ */
+int ffa_load_floor(int precision, int batch_size, int head_num, int head_dim, int max_seq_len, int t,
+                   const void* k_cache, const void* v_cache, const int* seq_lengths,
+                   int right_or_no_padding, const ffa_launch_plan* plan, void* sink, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

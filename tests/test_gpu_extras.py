@@ -527,3 +527,35 @@ def test_alternating_pruned_and_exact_calls_on_one_object():
         assert np.isfinite(got).all(), i
         assert np.abs(got - want).max() <= 1e-3 + 3e-4, (i, p)
     assert (capi.FFA_LAUNCH_WORKGROUP, False) in plans and (capi.FFA_LAUNCH_SPLIT, True) in plans, plans
+
+
+def test_load_floor_probe_runs_every_split_plan_and_touches_nothing():
+    """ffa_load_floor (the measurement aid behind bench.py's `load_floor_us`): every split plan with
+    one lane per key and 2 / 4 / 8 waves launches, the caches and the sink stay as they were (the
+    probe only loads), other plans are refused before anything is launched."""
+    lib = capi.load()
+    for prec, Dh in ((16, 64), (16, 80), (16, 256), (32, 64), (32, 128)):
+        B, H, L, Lmax = 2, 5, 700, 768
+        tdt = torch.float16 if prec == 16 else torch.float32
+        x = 16 // (prec // 8)
+        g = torch.Generator(device="cuda:0").manual_seed(prec + Dh)
+        kc = torch.randn(B, H, Dh // x, Lmax, x, device="cuda:0", generator=g).to(tdt)
+        vc = torch.randn(B, H, Lmax, Dh, device="cuda:0", generator=g).to(tdt)
+        kc0, vc0 = kc.clone(), vc.clone()
+        sink = torch.full((4,), 7, dtype=torch.int32, device="cuda:0")
+        ntiles = L // 64 + 1
+        for waves in (2, 4, 8):
+            for n_splits, whole in ((1, B * H), (3, 0), (4, 0), (11, 0)):
+                tps = -(-ntiles // n_splits)
+                plan = capi.make_plan(capi.FFA_LAUNCH_SPLIT, waves, -(-ntiles // tps), tps, 0, whole)
+                _say("load floor", prec, Dh, plan)
+                rc = lib.ffa_load_floor(prec, B, H, Dh, Lmax, L, ptr(kc), ptr(vc), None, 1, C.byref(plan), ptr(sink), None)
+                assert rc == capi.FFA_OK, capi.STATUS_NAMES.get(rc, rc)
+        torch.cuda.synchronize()
+        assert torch.equal(kc, kc0) and torch.equal(vc, vc0) and bool((sink == 7).all())
+        for bad in (capi.make_plan(capi.FFA_LAUNCH_WORKGROUP, 4, 1, ntiles),
+                    capi.make_plan(capi.FFA_LAUNCH_SPLIT, 3, 1, ntiles, 0, B * H),
+                    capi.make_plan(capi.FFA_LAUNCH_TWO_PASS, 4, 2, -(-ntiles // 2))):
+            rc = lib.ffa_load_floor(prec, B, H, Dh, Lmax, L, ptr(kc), ptr(vc), None, 1, C.byref(bad), ptr(sink), None)
+            assert rc == capi.FFA_ERR_PLAN, capi.STATUS_NAMES.get(rc, rc)
+        assert lib.ffa_load_floor(prec, B, H, Dh, Lmax, L, ptr(kc), ptr(vc), None, 1, None, ptr(sink), None) == capi.FFA_ERR_NULL_POINTER
