@@ -194,67 +194,141 @@ __device__ __forceinline__ void store_pair(bf16_t* p, float2 v) {
 // then once to T.  The reference does the same sums and products in fp32 (utils.h:1137-1156)
 // after adding the bias in T (attention.cu:870-873).
 //
-// In two steps, so that the loads of a wave's first tile can go out between them: the raw pairs
-// are loaded first (small loads at the head of the queue), the arithmetic -- an fp64 exp2 and
-// sincos per pair -- runs while the tile is on its way.
+// The wave that transforms a token does so in this order: the loads of the raw q pairs (their
+// address is among the preloaded kernel arguments, so they leave before the argument block has
+// been read), then the loads that need the argument block (k, v, the biases), then the angles --
+// an fp64 exp2, sine and cosine per pair, while all of those loads are on their way -- then q',
+// which the other waves of the workgroup are waiting for at a barrier, and only after the barrier
+// k' and v', which nobody but the transforming wave reads.
 template <typename T, int DH>
 struct RawToken {
     static constexpr int N = (DH / 2 + kWave - 1) / kWave;  // pairs per lane
     using Bits = typename PairBits<T>::type;
     Bits q[N], k[N], v[N], qb[N], kb[N], vb[N];
+    double sn[N], cs[N];  // sine and cosine of the pair's angle (0 and 1 outside the rotary part)
 };
 
 template <typename T, int DH>
-__device__ __forceinline__ RawToken<T, DH> token_raw_load(const DecodeParams& P, int bh, int h, bool with_kv, int lane) {
+__device__ __forceinline__ void token_raw_load(RawToken<T, DH>& r, const DecodeParams& P, int bh, bool with_kv, int lane) {
     using R = RawToken<T, DH>;
     using Bits = typename R::Bits;
-    R r;
+    auto ld = [](const void* base, size_t off) { return *reinterpret_cast<const Bits*>(static_cast<const char*>(base) + off); };
+#pragma unroll
+    for (int i = 0; i < R::N; ++i) {
+        const int z = min(lane + i * kWave, DH / 2 - 1);
+        r.q[i] = ld(P.q, ((size_t)bh * DH + 2 * z) * sizeof(T));
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    // Everything else the transform reads from the argument block, asked for in one batch (the
+    // compiler otherwise fetches each field in front of its first use: three round trips in a row).
+    asm volatile("" ::"s"(P.H), "s"(P.k), "s"(P.v), "s"(P.q_bias), "s"(P.k_bias), "s"(P.v_bias), "s"(P.rotary_dim),
+                 "s"(P.rotary_coef));
+    // Every load below is issued whatever is present (an absent operand reads q once more and
+    // the value is never looked at): with a fixed number of loads in flight the wait in front of
+    // q' is for q alone, not for the last load issued.
+    const int h = bh % P.H;
+    const void* qb = P.q_bias ? P.q_bias : P.q;
+    const void* kb = P.k_bias ? P.k_bias : P.q;
+    const void* vb = P.v_bias ? P.v_bias : P.q;
+    const void* k = with_kv ? P.k : P.q;
+    const void* v = with_kv ? P.v : P.q;
 #pragma unroll
     for (int i = 0; i < R::N; ++i) {
         const int z = min(lane + i * kWave, DH / 2 - 1);
         const size_t e = ((size_t)bh * DH + 2 * z) * sizeof(T), eb = ((size_t)h * DH + 2 * z) * sizeof(T);
-        auto ld = [](const void* base, size_t off) { return *reinterpret_cast<const Bits*>(static_cast<const char*>(base) + off); };
-        r.q[i] = ld(P.q, e);
-        r.k[i] = r.v[i] = r.qb[i] = r.kb[i] = r.vb[i] = Bits{};
-        if (P.q_bias) r.qb[i] = ld(P.q_bias, eb);
-        if (with_kv) {
-            r.k[i] = ld(P.k, e);
-            r.v[i] = ld(P.v, e);
-            if (P.k_bias) r.kb[i] = ld(P.k_bias, eb);
-            if (P.v_bias) r.vb[i] = ld(P.v_bias, eb);
-        }
+        r.qb[i] = ld(qb, P.q_bias ? eb : e);
+        r.k[i] = ld(k, e);
+        r.v[i] = ld(v, e);
+        r.kb[i] = ld(kb, P.k_bias ? eb : e);
+        r.vb[i] = ld(vb, P.v_bias ? eb : e);
     }
-    return r;
+    __builtin_amdgcn_sched_barrier(0);
 }
 
-// The results land in LDS in element order (s_q always, s_k and s_v only with `with_kv`, which
-// the token wave passes).
+// Sine and cosine of an fp64 angle 0 <= a < 2^31, to about one ulp: the quadrant from
+// k = rint(a * 2/pi), the remainder by two fused multiply-adds against pi/2 split in two (the first
+// is exact: a and k * P1 cancel to a multiple of 2^-52 below 2), then the classic minimax
+// polynomials on [-pi/4, pi/4].  Some fifty fp64 instructions without a branch, where the library's
+// sincos spends several hundred (its large-argument path, taken by some lanes of every wave, and
+// the divergence around it).
+__device__ __forceinline__ void sincos_reduced(double a, double* sn, double* cs) {
+    const double k = __builtin_rint(a * 0.63661977236758138);          // 2 / pi
+    double r = __builtin_fma(-k, 1.5707963267948966, a);               // pi / 2, rounded
+    r = __builtin_fma(-k, 6.123233995736766e-17, r);                   // pi / 2 - the above
+    const double z = r * r;
+    double ps = 1.58969099521155010221e-10;
+    ps = __builtin_fma(ps, z, -2.50507602534068634195e-08);
+    ps = __builtin_fma(ps, z, 2.75573137070700676789e-06);
+    ps = __builtin_fma(ps, z, -1.98412698298579493134e-04);
+    ps = __builtin_fma(ps, z, 8.33333333332248946124e-03);
+    ps = __builtin_fma(ps, z, -1.66666666666666324348e-01);
+    const double s0 = __builtin_fma(r * z, ps, r);
+    double pc = -1.13596475577881948265e-11;
+    pc = __builtin_fma(pc, z, 2.08757232129817482790e-09);
+    pc = __builtin_fma(pc, z, -2.75573143513906633035e-07);
+    pc = __builtin_fma(pc, z, 2.48015872894767294178e-05);
+    pc = __builtin_fma(pc, z, -1.38888888888741095749e-03);
+    pc = __builtin_fma(pc, z, 4.16666666666666019037e-02);
+    const double c0 = __builtin_fma(z * z, pc, __builtin_fma(-0.5, z, 1.0));
+    const int quadrant = (int)(long long)k & 3;
+    const double s1 = (quadrant & 1) ? c0 : s0, c1 = (quadrant & 1) ? s0 : c0;
+    *sn = (quadrant & 2) ? -s1 : s1;
+    *cs = ((quadrant + 1) & 2) ? -c1 : c1;
+}
+
+// Keeps the compiler from looking at a loaded pair before this point.
+__device__ __forceinline__ void pin_pair(uint32_t& x) { asm volatile("" : "+v"(x)); }
+__device__ __forceinline__ void pin_pair(uint2& x) { asm volatile("" : "+v"(x.x), "+v"(x.y)); }
+
+// The angles of the lane's pairs.  They depend on the position alone.  The empty asm statements
+// here and in pin_pair are volatile, hence kept in sequence: the angles are complete before the
+// first raw pair is looked at.  Left to itself the compiler waits for the loads first and starts
+// on the exp2, sine and cosine afterwards.
 template <typename T, int DH>
-__device__ __forceinline__ void transform_token(const DecodeParams& P, const RawToken<T, DH>& r, int pos, bool with_kv,
-                                                T* s_q, T* s_k, T* s_v, int lane) {
+__device__ __forceinline__ void token_angles(RawToken<T, DH>& r, const DecodeParams& P, int pos, int lane) {
     using R = RawToken<T, DH>;
 #pragma unroll
     for (int i = 0; i < R::N; ++i) {
         const int z = lane + i * kWave;
-        if (z >= DH / 2) break;
-        double2 q = widen_pair(r.q[i], T{}), k = widen_pair(r.k[i], T{}), v = widen_pair(r.v[i], T{});
-        // An absent bias was loaded as zero bits: adding it changes nothing.
-        const double2 qb = widen_pair(r.qb[i], T{}), kb = widen_pair(r.kb[i], T{}), vb = widen_pair(r.vb[i], T{});
-        q.x += qb.x; q.y += qb.y;
-        k.x += kb.x; k.y += kb.y;
-        v.x += vb.x; v.y += vb.y;
-        if (2 * z < P.rotary_dim) {
+        r.sn[i] = 0.0;
+        r.cs[i] = 1.0;
+        if (z < DH / 2 && 2 * z < P.rotary_dim) {
             const double angle = (double)pos * exp2((double)z * P.rotary_coef);
-            double sn, cs;
-            sincos(angle, &sn, &cs);
-            q = make_double2(cs * q.x - sn * q.y, cs * q.y + sn * q.x);
-            k = make_double2(cs * k.x - sn * k.y, cs * k.y + sn * k.x);
+            sincos_reduced(angle, &r.sn[i], &r.cs[i]);
         }
-        store_pair(s_q + 2 * z, make_float2((float)q.x, (float)q.y));
-        if (with_kv) {
-            store_pair(s_k + 2 * z, make_float2((float)k.x, (float)k.y));
-            store_pair(s_v + 2 * z, make_float2((float)v.x, (float)v.y));
+        asm volatile("" : "+v"(r.sn[i]), "+v"(r.cs[i]));
+    }
+}
+
+// x (+ bias, when there is one), rotated where `rotate`, rounded to fp32 and then once to T, into
+// LDS in element order.
+template <typename T, int DH>
+__device__ __forceinline__ void token_finish(RawToken<T, DH>& r, const DecodeParams& P, typename RawToken<T, DH>::Bits (&x)[RawToken<T, DH>::N],
+                                             typename RawToken<T, DH>::Bits (&bias)[RawToken<T, DH>::N], bool has_bias, bool rotate,
+                                             T* dst, int lane) {
+    using R = RawToken<T, DH>;
+    double2 a[R::N];
+#pragma unroll
+    for (int i = 0; i < R::N; ++i) {
+        pin_pair(x[i]);
+        a[i] = widen_pair(x[i], T{});
+    }
+    if (has_bias) {
+#pragma unroll
+        for (int i = 0; i < R::N; ++i) {
+            pin_pair(bias[i]);
+            const double2 ab = widen_pair(bias[i], T{});
+            a[i].x += ab.x;
+            a[i].y += ab.y;
         }
+    }
+#pragma unroll
+    for (int i = 0; i < R::N; ++i) {
+        const int z = lane + i * kWave;
+        if (z >= DH / 2) break;
+        double2 w = a[i];
+        if (rotate && 2 * z < P.rotary_dim) w = make_double2(r.cs[i] * w.x - r.sn[i] * w.y, r.cs[i] * w.y + r.sn[i] * w.x);
+        store_pair(dst + 2 * z, make_float2((float)w.x, (float)w.y));
     }
 }
 
@@ -266,26 +340,36 @@ struct alignas(16) TokenLds {
     uint4 v[Geo<T, DH>::NCH];
 };
 
-// q of the pair, ready for the dot products of the calling wave.  Every wave calls this.
-// Returns true when the dot products are to read q from LDS (s.q): wide heads, and every head
-// after a transform.  Otherwise q sits in SGPR-resident registers (q_reg), loaded straight from
-// memory through scalar loads.  With a transform every wave computes the transformed q itself
-// (identical values from every wave, so no workgroup barrier is needed before a wave reads what
-// it wrote) and, if it is the token wave, k' and v' as well.  The two sources are kept apart all
-// the way into the tile code: a register array fed from two places costs the plain path its
-// wide scalar loads.
+// q of the pair, ready for the dot products of the calling wave.  Every wave of the workgroup calls
+// this at the same point.  Returns true when the dot products are to read q from LDS (s.q): wide
+// heads, and every head after a transform.  Otherwise q sits in SGPR-resident registers (q_reg),
+// loaded straight from memory through scalar loads.  With a transform ONE wave (`compute`) does the
+// arithmetic -- q' and, `with_kv`, k' and v' -- and a workgroup barrier hands the result to the
+// others: the fp64 sine and cosine are some hundreds of instructions, and five waves doing them
+// side by side on four SIMDs kept every wave from its first tile for longer than the tile's
+// loads take.  The two sources of q are kept apart all the way into the tile code: a register
+// array fed from two places costs the plain path its wide scalar loads.
 template <typename T, int DH, bool XFORM>
-__device__ __forceinline__ bool setup_q(const DecodeParams& P, int bh, int h, int tlen, int first, bool token_wave,
-                                        TokenLds<T, DH>& s, uint4 (&q_reg)[Geo<T, DH>::QREG], int lane) {
+__device__ __forceinline__ bool setup_q(const DecodeParams& P, int bh, int tlen, int first, bool compute,
+                                        bool with_kv, TokenLds<T, DH>& s, uint4 (&q_reg)[Geo<T, DH>::QREG], int lane) {
     using G = Geo<T, DH>;
     const uint4* qg = reinterpret_cast<const uint4*>(reinterpret_cast<const char*>(P.q) + (size_t)bh * DH * sizeof(T));
     if constexpr (XFORM) {
-        const RawToken<T, DH> raw = token_raw_load<T, DH>(P, bh, h, token_wave, lane);
-        transform_token<T, DH>(P, raw, max(tlen - first, 0), token_wave, reinterpret_cast<T*>(s.q),
-                               reinterpret_cast<T*>(s.k), reinterpret_cast<T*>(s.v), lane);
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-        __builtin_amdgcn_wave_barrier();
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        RawToken<T, DH> raw;
+        if (compute) {
+            token_raw_load<T, DH>(raw, P, bh, with_kv, lane);
+            token_angles<T, DH>(raw, P, max(tlen - first, 0), lane);
+            token_finish<T, DH>(raw, P, raw.q, raw.qb, P.q_bias != nullptr, true, reinterpret_cast<T*>(s.q), lane);
+        }
+        __syncthreads();
+        if (compute && with_kv) {
+            token_finish<T, DH>(raw, P, raw.k, raw.kb, P.k_bias != nullptr, true, reinterpret_cast<T*>(s.k), lane);
+            token_finish<T, DH>(raw, P, raw.v, raw.vb, P.v_bias != nullptr, false, reinterpret_cast<T*>(s.v), lane);
+            // Read back by this wave alone.
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        }
         return true;
     }
     if constexpr (G::Q_LDS) {
@@ -302,18 +386,6 @@ __device__ __forceinline__ bool setup_q(const DecodeParams& P, int bh, int h, in
     }
 }
 
-// The transform of q alone, by a tile wave, from raw pairs it loaded before its first tile: the
-// arithmetic runs while that tile is on its way.
-template <typename T, int DH>
-__device__ __forceinline__ void transform_q_only(const DecodeParams& P, const RawToken<T, DH>& raw, int tlen, int first,
-                                                 TokenLds<T, DH>& s, int lane) {
-    transform_token<T, DH>(P, raw, max(tlen - first, 0), /*with_kv=*/false, reinterpret_cast<T*>(s.q),
-                           reinterpret_cast<T*>(s.k), reinterpret_cast<T*>(s.v), lane);
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    __builtin_amdgcn_wave_barrier();
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-}
-
 // The new token in the token wave's registers: lane c < NCH holds 16-byte chunk c of q, k, v
 // (after the transform, if any).
 struct TokenRegs {
@@ -324,7 +396,7 @@ __device__ __forceinline__ TokenRegs token_load(const DecodeParams& P, int bh, c
     constexpr int NCH = Geo<T, DH>::NCH;
     const int c = lane < NCH ? lane : 0;
     TokenRegs r;
-    if constexpr (XFORM) {  // setup_q of this wave has put them in LDS
+    if constexpr (XFORM) {  // the transform has put them in LDS
         r.q = s.q[c];
         r.k = s.k[c];
         r.v = s.v[c];
@@ -547,12 +619,10 @@ __device__ __forceinline__ void queue_drain(float (&acc)[Elem<T>::X], SurvivorQu
 // write turns memory channels around under the reads (measured at 320 pairs x 1000 keys: 0.1 us
 // per launch for 640 small stores).
 template <typename T, int DH, bool XFORM>
-__device__ __forceinline__ TokenRegs token_wave_state(const DecodeParams& P, int bh, int h, int tlen, int first,
+__device__ __forceinline__ TokenRegs token_wave_state(const DecodeParams& P, int bh, int tlen, int first,
                                                       TokenLds<T, DH>& s_tok, float& m_run, float& l_run,
                                                       float (&acc)[Elem<T>::X], int lane) {
     constexpr int NCH = Geo<T, DH>::NCH;
-    uint4 q_unused[Geo<T, DH>::QREG];
-    if constexpr (XFORM) (void)setup_q<T, DH, true>(P, bh, h, tlen, first, /*token_wave=*/true, s_tok, q_unused, lane);
     const TokenRegs tok = token_load<T, DH, XFORM>(P, bh, s_tok, lane);
     const float s = token_score<T, DH>(tok, lane);
     if (tlen >= first) {  // else the whole sample is masked up to and including the new slot
@@ -730,7 +800,7 @@ ffa_decode_split_kernel(HOT_PARAMS_DECL, const DecodeParams P_rest) {
     // cross-workgroup merges (a chain of memory round trips) finish in their shadow.
     const PieceOf piece(P, (int)blockIdx.x);
     const int bh = piece.bh, split = piece.split, n_splits = piece.n_splits;
-    const bool need_b = P.seq_lengths != nullptr || BEAM || XFORM;
+    const bool need_b = P.seq_lengths != nullptr || BEAM;
     const int b = need_b ? bh / P.H : 0;
 
     int tlen, first;
@@ -781,7 +851,14 @@ ffa_decode_split_kernel(HOT_PARAMS_DECL, const DecodeParams P_rest) {
     TokenRegs tok;
     const bool has_token = token_wave && split == n_splits - 1;
     if (token_wave) {
-        if (has_token) tok = token_wave_state<T, DH, XFORM>(P, bh, bh - b * P.H, tlen, first, s_tok, m_run, l_run, acc, lane);
+        if constexpr (XFORM) {
+            // The token wave of EVERY workgroup transforms q (k and v too where it holds the token)
+            // while the tile waves' first tiles are on their way; the barrier hands q' over.
+            uint4 q_unused[G::QREG];
+            (void)setup_q<T, DH, true>(P, bh, tlen, first, /*compute=*/true, /*with_kv=*/has_token, s_tok,
+                                       q_unused, lane);
+        }
+        if (has_token) tok = token_wave_state<T, DH, XFORM>(P, bh, tlen, first, s_tok, m_run, l_run, acc, lane);
     } else {
     uint4 q_reg[G::QREG];
 
@@ -872,21 +949,21 @@ ffa_decode_split_kernel(HOT_PARAMS_DECL, const DecodeParams P_rest) {
         }
     };
     if constexpr (XFORM) {
-        // With a transform: raw pairs of q first (small loads at the head of the queue), then the
-        // loads of the wave's first tile, then the fp64 arithmetic in the shadow of that tile.
-        if (wave < order.n) {
-            const RawToken<T, DH> raw = token_raw_load<T, DH>(P, bh, bh - b * P.H, /*with_kv=*/false, lane);
-            const int tile = order.at(wave);
-            const int src = beams.beam(min(tile * kWave + lane, last_key), tlen);
-            uint4 kv[CG], vv[VG];
-            load_tile(kv, vv, tile, src);
-            __builtin_amdgcn_sched_barrier(0);
-            transform_q_only<T, DH>(P, raw, tlen, first, s_tok, lane);
+        // With a transform: the loads of the wave's first tile go out, then the wave meets the
+        // token wave, which has transformed q in the meantime, at the workgroup barrier.
+        const bool has_tile = wave < order.n;
+        const int tile = has_tile ? order.at(wave) : 0;
+        const int src = has_tile ? beams.beam(min(tile * kWave + lane, last_key), tlen) : 0;
+        uint4 kv[CG], vv[VG];
+        if (has_tile) load_tile(kv, vv, tile, src);
+        __builtin_amdgcn_sched_barrier(0);
+        __syncthreads();
+        if (has_tile) {
             compute_tile(std::true_type{}, kv, vv, tile, src);
             walk_tiles(std::true_type{}, wave + NW);
         }
     } else {
-        const bool q_in_lds = setup_q<T, DH, false>(P, bh, 0, tlen, first, /*token_wave=*/false, s_tok, q_reg, lane);
+        const bool q_in_lds = setup_q<T, DH, false>(P, bh, tlen, first, false, false, s_tok, q_reg, lane);
         if constexpr (G::Q_LDS) {
             (void)q_in_lds;
             walk_tiles(std::true_type{}, wave);
@@ -930,7 +1007,7 @@ ffa_decode_split_tpk_kernel(HOT_PARAMS_DECL, const DecodeParams P_rest) {
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const PieceOf piece(P, (int)blockIdx.x);
     const int bh = piece.bh, split = piece.split, n_splits = piece.n_splits;
-    const bool need_b = P.seq_lengths != nullptr || BEAM || XFORM;
+    const bool need_b = P.seq_lengths != nullptr || BEAM;
     const int b = need_b ? bh / P.H : 0;
     int tlen, first;
     step_bounds(P, b, tlen, first);
@@ -976,7 +1053,12 @@ ffa_decode_split_tpk_kernel(HOT_PARAMS_DECL, const DecodeParams P_rest) {
     TokenRegs tok;
     const bool has_token = token_wave && split == n_splits - 1;
     if (token_wave) {
-        if (has_token) tok = token_wave_state<T, DH, XFORM>(P, bh, bh - b * P.H, tlen, first, s_tok, m_run, l_run, acc, lane);
+        if constexpr (XFORM) {  // as in ffa_decode_split_kernel
+            uint4 q_unused[G::QREG];
+            (void)setup_q<T, DH, true>(P, bh, tlen, first, /*compute=*/true, /*with_kv=*/has_token, s_tok,
+                                       q_unused, lane);
+        }
+        if (has_token) tok = token_wave_state<T, DH, XFORM>(P, bh, tlen, first, s_tok, m_run, l_run, acc, lane);
     } else {
     uint4 q_reg[NK];  // this lane's share of q: chunks [part*NK, part*NK + NK)
     auto compute_tile = [&](uint4 (&kv)[NK], uint4 (&vv)[NV], int tile) {
@@ -1019,15 +1101,15 @@ ffa_decode_split_tpk_kernel(HOT_PARAMS_DECL, const DecodeParams P_rest) {
         }
     };
     if constexpr (XFORM) {
-        // As in ffa_decode_split_kernel: raw pairs, first tile's loads, arithmetic in their shadow.
-        if (wave < order.n) {
-            const RawToken<T, DH> raw = token_raw_load<T, DH>(P, bh, bh - b * P.H, /*with_kv=*/false, lane);
-            const int tile = order.at(wave);
-            const int src = beams.beam(min(tile * KPT + kl, last_key), tlen);
-            uint4 kv[NK], vv[NV];
-            load_tile(kv, vv, tile, src);
-            __builtin_amdgcn_sched_barrier(0);
-            transform_q_only<T, DH>(P, raw, tlen, first, s_tok, lane);
+        // As in ffa_decode_split_kernel: first tile's loads, then the barrier behind which q' waits.
+        const bool has_tile = wave < order.n;
+        const int tile = has_tile ? order.at(wave) : 0;
+        const int src = has_tile ? beams.beam(min(tile * KPT + kl, last_key), tlen) : 0;
+        uint4 kv[NK], vv[NV];
+        if (has_tile) load_tile(kv, vv, tile, src);
+        __builtin_amdgcn_sched_barrier(0);
+        __syncthreads();
+        if (has_tile) {
 #pragma unroll
             for (int i = 0; i < NK; ++i) q_reg[i] = s_tok.q[part * NK + i];
             compute_tile(kv, vv, tile);
@@ -1035,7 +1117,7 @@ ffa_decode_split_tpk_kernel(HOT_PARAMS_DECL, const DecodeParams P_rest) {
         }
     } else {
         uint4 q_full[G::QREG];
-        const bool q_in_lds = setup_q<T, DH, false>(P, bh, 0, tlen, first, /*token_wave=*/false, s_tok, q_full, lane);
+        const bool q_in_lds = setup_q<T, DH, false>(P, bh, tlen, first, false, false, s_tok, q_full, lane);
         if (q_in_lds) {
 #pragma unroll
             for (int i = 0; i < NK; ++i) q_reg[i] = s_tok.q[part * NK + i];
@@ -1158,7 +1240,7 @@ __global__ void __launch_bounds__(NW * 64) ffa_decode_wg_kernel(HOT_PARAMS_DECL,
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int bh = blockIdx.x;
-    const int b = bh / P.H;
+    const int b = (P.seq_lengths != nullptr || BEAM) ? bh / P.H : 0;  // nobody else asks for it
 
     int tlen, first;
     step_bounds(P, b, tlen, first);
@@ -1171,7 +1253,8 @@ __global__ void __launch_bounds__(NW * 64) ffa_decode_wg_kernel(HOT_PARAMS_DECL,
 
     const bool token_wave = wave == 0;
     uint4 q_reg[G::QREG];
-    const bool q_in_lds = setup_q<T, DH, XFORM>(P, bh, bh - b * P.H, tlen, first, token_wave, s_tok, q_reg, lane);
+    const bool q_in_lds = setup_q<T, DH, XFORM>(P, bh, tlen, first, /*compute=*/token_wave, /*with_kv=*/true,
+                                                s_tok, q_reg, lane);
     TokenRegs tok;
     if (token_wave) tok = token_load<T, DH, XFORM>(P, bh, s_tok, lane);
 
@@ -1358,7 +1441,7 @@ __global__ void __launch_bounds__(NW * 64) ffa_scores_kernel(HOT_PARAMS_DECL, co
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const unsigned pair = pair_of(P, blockIdx.x);
     const int bh = (int)pair, split = (int)(blockIdx.x - pair * (unsigned)P.n_splits);
-    const int b = bh / P.H;
+    const int b = (P.seq_lengths != nullptr || BEAM) ? bh / P.H : 0;  // nobody else asks for it
     int tlen, first;
     step_bounds(P, b, tlen, first);
 
@@ -1368,7 +1451,9 @@ __global__ void __launch_bounds__(NW * 64) ffa_scores_kernel(HOT_PARAMS_DECL, co
 
     const bool token_wave = split == P.n_splits - 1 && wave == 0;
     uint4 q_reg[G::QREG];
-    const bool q_in_lds = setup_q<T, DH, XFORM>(P, bh, bh - b * P.H, tlen, first, token_wave, s_tok, q_reg, lane);
+    // With a transform, wave 0 of every piece transforms q; the piece that holds the token also k and v.
+    const bool q_in_lds = setup_q<T, DH, XFORM>(P, bh, tlen, first, /*compute=*/wave == 0,
+                                                /*with_kv=*/token_wave, s_tok, q_reg, lane);
     TokenRegs tok;
     if (token_wave) tok = token_load<T, DH, XFORM>(P, bh, s_tok, lane);
 
@@ -1451,7 +1536,7 @@ __global__ void __launch_bounds__(NW * 64) ffa_pruned_pv_kernel(PV_HOT_PARAMS_DE
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const unsigned pair = pair_of(P, blockIdx.x);
     const int bh = (int)pair, split = (int)(blockIdx.x - pair * (unsigned)P.n_splits);
-    const int b = bh / P.H;
+    const int b = (P.seq_lengths != nullptr || BEAM) ? bh / P.H : 0;  // nobody else asks for it
     int tlen, first;
     step_bounds(P, b, tlen, first);
 
