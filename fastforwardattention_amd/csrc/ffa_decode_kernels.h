@@ -194,12 +194,14 @@ __device__ __forceinline__ void store_pair(bf16_t* p, float2 v) {
 // then once to T.  The reference does the same sums and products in fp32 (utils.h:1137-1156)
 // after adding the bias in T (attention.cu:870-873).
 //
-// The wave that transforms a token does so in this order: the loads of the raw q pairs (their
-// address is among the preloaded kernel arguments, so they leave before the argument block has
-// been read), then the loads that need the argument block (k, v, the biases), then the angles --
-// an fp64 exp2, sine and cosine per pair, while all of those loads are on their way -- then q',
-// which the other waves of the workgroup are waiting for at a barrier, and only after the barrier
-// k' and v', which nobody but the transforming wave reads.
+// One wave of a workgroup -- the publisher -- computes the angles (an fp64 exp2, sine and cosine
+// per pair: some hundreds of instructions) and leaves their cosines and sines in LDS, together
+// with the q bias, ahead of a workgroup barrier.  They depend on the position alone, so the
+// barrier is reached while the first cache tiles are still on their way.  Every wave that needs
+// q' then rotates its own copy of q (a dozen fp64 instructions), which it loaded as the very
+// first thing it did: the address of q is among the preloaded kernel arguments, so that load
+// leaves before the argument block has been read and returns before the wave's first tile.  The
+// wave that appends the token does the same for k and v.
 template <typename T, int DH>
 struct RawToken {
     static constexpr int N = (DH / 2 + kWave - 1) / kWave;  // pairs per lane
@@ -208,24 +210,40 @@ struct RawToken {
     double sn[N], cs[N];  // sine and cosine of the pair's angle (0 and 1 outside the rotary part)
 };
 
+// What the publisher leaves in LDS for the other waves of the workgroup.
+template <typename T, int DH, bool XFORM>
+struct alignas(16) AngleLds {
+    double2 cs_sn[XFORM ? DH / 2 : 1];
+    typename PairBits<T>::type q_bias[XFORM ? DH / 2 : 1];  // zero bits when there is none
+};
+
 template <typename T, int DH>
-__device__ __forceinline__ void token_raw_load(RawToken<T, DH>& r, const DecodeParams& P, int bh, bool with_kv, int lane) {
-    using R = RawToken<T, DH>;
-    using Bits = typename R::Bits;
-    auto ld = [](const void* base, size_t off) { return *reinterpret_cast<const Bits*>(static_cast<const char*>(base) + off); };
+__device__ __forceinline__ typename PairBits<T>::type load_pair(const void* base, size_t off) {
+    return *reinterpret_cast<const typename PairBits<T>::type*>(static_cast<const char*>(base) + off);
+}
+
+// First thing a wave does: its pairs of q.
+template <typename T, int DH>
+__device__ __forceinline__ void token_load_q(RawToken<T, DH>& r, const DecodeParams& P, int bh, int lane) {
 #pragma unroll
-    for (int i = 0; i < R::N; ++i) {
+    for (int i = 0; i < RawToken<T, DH>::N; ++i) {
         const int z = min(lane + i * kWave, DH / 2 - 1);
-        r.q[i] = ld(P.q, ((size_t)bh * DH + 2 * z) * sizeof(T));
+        r.q[i] = load_pair<T, DH>(P.q, ((size_t)bh * DH + 2 * z) * sizeof(T));
     }
     __builtin_amdgcn_sched_barrier(0);
-    // Everything else the transform reads from the argument block, asked for in one batch (the
+}
+
+// The publisher's other loads: the q bias, and with `with_kv` k, v and their biases.
+template <typename T, int DH>
+__device__ __forceinline__ void token_load_rest(RawToken<T, DH>& r, const DecodeParams& P, int bh, bool with_kv, int lane) {
+    using R = RawToken<T, DH>;
+    // Everything the transform reads from the argument block, asked for in one batch (the
     // compiler otherwise fetches each field in front of its first use: three round trips in a row).
     asm volatile("" ::"s"(P.H), "s"(P.k), "s"(P.v), "s"(P.q_bias), "s"(P.k_bias), "s"(P.v_bias), "s"(P.rotary_dim),
                  "s"(P.rotary_coef));
     // Every load below is issued whatever is present (an absent operand reads q once more and
-    // the value is never looked at): with a fixed number of loads in flight the wait in front of
-    // q' is for q alone, not for the last load issued.
+    // the value is never looked at): with a fixed number of loads in flight each wait is for the
+    // operand it names, not for the last load issued.
     const int h = bh % P.H;
     const void* qb = P.q_bias ? P.q_bias : P.q;
     const void* kb = P.k_bias ? P.k_bias : P.q;
@@ -236,11 +254,11 @@ __device__ __forceinline__ void token_raw_load(RawToken<T, DH>& r, const DecodeP
     for (int i = 0; i < R::N; ++i) {
         const int z = min(lane + i * kWave, DH / 2 - 1);
         const size_t e = ((size_t)bh * DH + 2 * z) * sizeof(T), eb = ((size_t)h * DH + 2 * z) * sizeof(T);
-        r.qb[i] = ld(qb, P.q_bias ? eb : e);
-        r.k[i] = ld(k, e);
-        r.v[i] = ld(v, e);
-        r.kb[i] = ld(kb, P.k_bias ? eb : e);
-        r.vb[i] = ld(vb, P.v_bias ? eb : e);
+        r.qb[i] = load_pair<T, DH>(qb, P.q_bias ? eb : e);
+        r.k[i] = load_pair<T, DH>(k, e);
+        r.v[i] = load_pair<T, DH>(v, e);
+        r.kb[i] = load_pair<T, DH>(kb, P.k_bias ? eb : e);
+        r.vb[i] = load_pair<T, DH>(vb, P.v_bias ? eb : e);
     }
     __builtin_amdgcn_sched_barrier(0);
 }
@@ -340,38 +358,73 @@ struct alignas(16) TokenLds {
     uint4 v[Geo<T, DH>::NCH];
 };
 
-// q of the pair, ready for the dot products of the calling wave.  Every wave of the workgroup calls
-// this at the same point.  Returns true when the dot products are to read q from LDS (s.q): wide
-// heads, and every head after a transform.  Otherwise q sits in SGPR-resident registers (q_reg),
-// loaded straight from memory through scalar loads.  With a transform ONE wave (`compute`) does the
-// arithmetic -- q' and, `with_kv`, k' and v' -- and a workgroup barrier hands the result to the
-// others: the fp64 sine and cosine are some hundreds of instructions, and five waves doing them
-// side by side on four SIMDs kept every wave from its first tile for longer than the tile's
-// loads take.  The two sources of q are kept apart all the way into the tile code: a register
-// array fed from two places costs the plain path its wide scalar loads.
-template <typename T, int DH, bool XFORM>
-__device__ __forceinline__ bool setup_q(const DecodeParams& P, int bh, int tlen, int first, bool compute,
-                                        bool with_kv, TokenLds<T, DH>& s, uint4 (&q_reg)[Geo<T, DH>::QREG], int lane) {
+// The transform of a workgroup, first half, called by every wave as the first thing it does
+// (callers then issue the loads of their first tile, then call xform_end).  `needs_q`: the wave
+// will read q' (tile waves, and the wave that appends the token).  `publisher`: the one wave that
+// computes the angles; `with_kv`: it also transforms k and v (it holds the token).
+template <typename T, int DH>
+__device__ __forceinline__ void xform_begin(RawToken<T, DH>& r, const DecodeParams& P, int bh, int tlen, int first,
+                                            bool needs_q, bool publisher, bool with_kv, AngleLds<T, DH, true>& s_ang,
+                                            int lane) {
+    using R = RawToken<T, DH>;
+    if (needs_q) token_load_q<T, DH>(r, P, bh, lane);
+    if (publisher) {
+        token_load_rest<T, DH>(r, P, bh, with_kv, lane);
+        token_angles<T, DH>(r, P, max(tlen - first, 0), lane);
+        const bool has_bias = P.q_bias != nullptr;
+#pragma unroll
+        for (int i = 0; i < R::N; ++i) {
+            const int z = lane + i * kWave;
+            if (z >= DH / 2) break;
+            s_ang.cs_sn[z] = make_double2(r.cs[i], r.sn[i]);
+            typename R::Bits bits{};
+            if (has_bias) {
+                pin_pair(r.qb[i]);
+                bits = r.qb[i];
+            }
+            s_ang.q_bias[z] = bits;
+        }
+    }
+}
+
+// Second half: the barrier behind which the angles wait, then q' (and k', v') into LDS.  Every
+// wave that needs q' writes the same values to the same place; a wave reads back only after its
+// own stores.
+template <typename T, int DH>
+__device__ __forceinline__ void xform_end(RawToken<T, DH>& r, const DecodeParams& P, bool needs_q, bool publisher,
+                                          bool with_kv, TokenLds<T, DH>& s, AngleLds<T, DH, true>& s_ang, int lane) {
+    using R = RawToken<T, DH>;
+    __syncthreads();
+    if (needs_q) {
+#pragma unroll
+        for (int i = 0; i < R::N; ++i) {
+            const int z = min(lane + i * kWave, DH / 2 - 1);
+            const double2 a = s_ang.cs_sn[z];
+            r.cs[i] = a.x;
+            r.sn[i] = a.y;
+            r.qb[i] = s_ang.q_bias[z];
+        }
+        token_finish<T, DH>(r, P, r.q, r.qb, true, true, reinterpret_cast<T*>(s.q), lane);
+    }
+    if (publisher && with_kv) {
+        token_finish<T, DH>(r, P, r.k, r.kb, P.k_bias != nullptr, true, reinterpret_cast<T*>(s.k), lane);
+        token_finish<T, DH>(r, P, r.v, r.vb, P.v_bias != nullptr, false, reinterpret_cast<T*>(s.v), lane);
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
+// q of the pair without a transform, ready for the dot products of the calling wave.  Returns
+// true when the dot products are to read q from LDS (s.q): wide heads.  Otherwise q sits in
+// SGPR-resident registers (q_reg), loaded straight from memory through scalar loads.  The two
+// sources of q are kept apart all the way into the tile code: a register array fed from two
+// places costs the plain path its wide scalar loads.
+template <typename T, int DH>
+__device__ __forceinline__ bool setup_q(const DecodeParams& P, int bh, TokenLds<T, DH>& s, uint4 (&q_reg)[Geo<T, DH>::QREG],
+                                        int lane) {
     using G = Geo<T, DH>;
     const uint4* qg = reinterpret_cast<const uint4*>(reinterpret_cast<const char*>(P.q) + (size_t)bh * DH * sizeof(T));
-    if constexpr (XFORM) {
-        RawToken<T, DH> raw;
-        if (compute) {
-            token_raw_load<T, DH>(raw, P, bh, with_kv, lane);
-            token_angles<T, DH>(raw, P, max(tlen - first, 0), lane);
-            token_finish<T, DH>(raw, P, raw.q, raw.qb, P.q_bias != nullptr, true, reinterpret_cast<T*>(s.q), lane);
-        }
-        __syncthreads();
-        if (compute && with_kv) {
-            token_finish<T, DH>(raw, P, raw.k, raw.kb, P.k_bias != nullptr, true, reinterpret_cast<T*>(s.k), lane);
-            token_finish<T, DH>(raw, P, raw.v, raw.vb, P.v_bias != nullptr, false, reinterpret_cast<T*>(s.v), lane);
-            // Read back by this wave alone.
-            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-            __builtin_amdgcn_wave_barrier();
-            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-        }
-        return true;
-    }
     if constexpr (G::Q_LDS) {
         // Every wave stores the same values; a wave reads back only after its own stores.
         if (lane < G::NCH) s.q[lane] = qg[lane];
@@ -790,6 +843,7 @@ ffa_decode_split_kernel(HOT_PARAMS_DECL, const DecodeParams P_rest) {
     __shared__ float s_p[NW][kWave];
     __shared__ MergeLds<T, DH, NW + 1> s_merge;
     __shared__ TokenLds<T, DH> s_tok;
+    __shared__ AngleLds<T, DH, XFORM> s_ang;
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform, and known to be so
@@ -852,11 +906,12 @@ ffa_decode_split_kernel(HOT_PARAMS_DECL, const DecodeParams P_rest) {
     const bool has_token = token_wave && split == n_splits - 1;
     if (token_wave) {
         if constexpr (XFORM) {
-            // The token wave of EVERY workgroup transforms q (k and v too where it holds the token)
-            // while the tile waves' first tiles are on their way; the barrier hands q' over.
-            uint4 q_unused[G::QREG];
-            (void)setup_q<T, DH, true>(P, bh, tlen, first, /*compute=*/true, /*with_kv=*/has_token, s_tok,
-                                       q_unused, lane);
+            // The token wave of EVERY workgroup publishes the angles while the tile waves' first
+            // tiles are on their way; where it holds the token it also transforms q, k and v.
+            RawToken<T, DH> raw;
+            xform_begin<T, DH>(raw, P, bh, tlen, first, /*needs_q=*/has_token, /*publisher=*/true, /*with_kv=*/has_token,
+                               s_ang, lane);
+            xform_end<T, DH>(raw, P, has_token, true, has_token, s_tok, s_ang, lane);
         }
         if (has_token) tok = token_wave_state<T, DH, XFORM>(P, bh, tlen, first, s_tok, m_run, l_run, acc, lane);
     } else {
@@ -949,21 +1004,27 @@ ffa_decode_split_kernel(HOT_PARAMS_DECL, const DecodeParams P_rest) {
         }
     };
     if constexpr (XFORM) {
-        // With a transform: the loads of the wave's first tile go out, then the wave meets the
-        // token wave, which has transformed q in the meantime, at the workgroup barrier.
+        // With a transform: the load of q, the loads of the wave's first tile, then the barrier
+        // behind which the token wave has left the angles, then q'.
+        // (The barrier stands in both branches: behind a join the compiler no longer knows how many
+        // loads follow that of q, and waits for all of them before it lets the wave look at q.)
         const bool has_tile = wave < order.n;
-        const int tile = has_tile ? order.at(wave) : 0;
-        const int src = has_tile ? beams.beam(min(tile * kWave + lane, last_key), tlen) : 0;
-        uint4 kv[CG], vv[VG];
-        if (has_tile) load_tile(kv, vv, tile, src);
-        __builtin_amdgcn_sched_barrier(0);
-        __syncthreads();
+        RawToken<T, DH> raw;
+        xform_begin<T, DH>(raw, P, bh, tlen, first, /*needs_q=*/has_tile, /*publisher=*/false, false, s_ang, lane);
         if (has_tile) {
+            const int tile = order.at(wave);
+            const int src = beams.beam(min(tile * kWave + lane, last_key), tlen);
+            uint4 kv[CG], vv[VG];
+            load_tile(kv, vv, tile, src);
+            __builtin_amdgcn_sched_barrier(0);
+            xform_end<T, DH>(raw, P, true, false, false, s_tok, s_ang, lane);
             compute_tile(std::true_type{}, kv, vv, tile, src);
             walk_tiles(std::true_type{}, wave + NW);
+        } else {
+            xform_end<T, DH>(raw, P, false, false, false, s_tok, s_ang, lane);
         }
     } else {
-        const bool q_in_lds = setup_q<T, DH, false>(P, bh, tlen, first, false, false, s_tok, q_reg, lane);
+        const bool q_in_lds = setup_q<T, DH>(P, bh, s_tok, q_reg, lane);
         if constexpr (G::Q_LDS) {
             (void)q_in_lds;
             walk_tiles(std::true_type{}, wave);
@@ -1002,6 +1063,7 @@ ffa_decode_split_tpk_kernel(HOT_PARAMS_DECL, const DecodeParams P_rest) {
     __shared__ float s_p[NW][KPT];
     __shared__ MergeLds<T, DH, NW + 1> s_merge;
     __shared__ TokenLds<T, DH> s_tok;
+    __shared__ AngleLds<T, DH, XFORM> s_ang;
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -1054,9 +1116,10 @@ ffa_decode_split_tpk_kernel(HOT_PARAMS_DECL, const DecodeParams P_rest) {
     const bool has_token = token_wave && split == n_splits - 1;
     if (token_wave) {
         if constexpr (XFORM) {  // as in ffa_decode_split_kernel
-            uint4 q_unused[G::QREG];
-            (void)setup_q<T, DH, true>(P, bh, tlen, first, /*compute=*/true, /*with_kv=*/has_token, s_tok,
-                                       q_unused, lane);
+            RawToken<T, DH> raw;
+            xform_begin<T, DH>(raw, P, bh, tlen, first, /*needs_q=*/has_token, /*publisher=*/true, /*with_kv=*/has_token,
+                               s_ang, lane);
+            xform_end<T, DH>(raw, P, has_token, true, has_token, s_tok, s_ang, lane);
         }
         if (has_token) tok = token_wave_state<T, DH, XFORM>(P, bh, tlen, first, s_tok, m_run, l_run, acc, lane);
     } else {
@@ -1101,23 +1164,27 @@ ffa_decode_split_tpk_kernel(HOT_PARAMS_DECL, const DecodeParams P_rest) {
         }
     };
     if constexpr (XFORM) {
-        // As in ffa_decode_split_kernel: first tile's loads, then the barrier behind which q' waits.
+        // As in ffa_decode_split_kernel: q, the first tile's loads, the barrier, q'.
         const bool has_tile = wave < order.n;
-        const int tile = has_tile ? order.at(wave) : 0;
-        const int src = has_tile ? beams.beam(min(tile * KPT + kl, last_key), tlen) : 0;
-        uint4 kv[NK], vv[NV];
-        if (has_tile) load_tile(kv, vv, tile, src);
-        __builtin_amdgcn_sched_barrier(0);
-        __syncthreads();
+        RawToken<T, DH> raw;
+        xform_begin<T, DH>(raw, P, bh, tlen, first, /*needs_q=*/has_tile, /*publisher=*/false, false, s_ang, lane);
         if (has_tile) {
+            const int tile = order.at(wave);
+            const int src = beams.beam(min(tile * KPT + kl, last_key), tlen);
+            uint4 kv[NK], vv[NV];
+            load_tile(kv, vv, tile, src);
+            __builtin_amdgcn_sched_barrier(0);
+            xform_end<T, DH>(raw, P, true, false, false, s_tok, s_ang, lane);
 #pragma unroll
             for (int i = 0; i < NK; ++i) q_reg[i] = s_tok.q[part * NK + i];
             compute_tile(kv, vv, tile);
             walk_tiles(wave + NW);
+        } else {
+            xform_end<T, DH>(raw, P, false, false, false, s_tok, s_ang, lane);
         }
     } else {
         uint4 q_full[G::QREG];
-        const bool q_in_lds = setup_q<T, DH, false>(P, bh, tlen, first, false, false, s_tok, q_full, lane);
+        const bool q_in_lds = setup_q<T, DH>(P, bh, s_tok, q_full, lane);
         if (q_in_lds) {
 #pragma unroll
             for (int i = 0; i < NK; ++i) q_reg[i] = s_tok.q[part * NK + i];
@@ -1235,6 +1302,7 @@ __global__ void __launch_bounds__(NW * 64) ffa_decode_wg_kernel(HOT_PARAMS_DECL,
     __shared__ float s_red[NW];
     __shared__ unsigned s_cnt[NW];
     __shared__ TokenLds<T, DH> s_tok;
+    __shared__ AngleLds<T, DH, XFORM> s_ang;
     __shared__ float s_qw[NW][2 * kWave];
     __shared__ int s_qr[NW][2 * kWave];
 
@@ -1253,8 +1321,14 @@ __global__ void __launch_bounds__(NW * 64) ffa_decode_wg_kernel(HOT_PARAMS_DECL,
 
     const bool token_wave = wave == 0;
     uint4 q_reg[G::QREG];
-    const bool q_in_lds = setup_q<T, DH, XFORM>(P, bh, tlen, first, /*compute=*/token_wave, /*with_kv=*/true,
-                                                s_tok, q_reg, lane);
+    bool q_in_lds = true;
+    if constexpr (XFORM) {
+        RawToken<T, DH> raw;
+        xform_begin<T, DH>(raw, P, bh, tlen, first, /*needs_q=*/true, /*publisher=*/token_wave, /*with_kv=*/true, s_ang, lane);
+        xform_end<T, DH>(raw, P, true, token_wave, true, s_tok, s_ang, lane);
+    } else {
+        q_in_lds = setup_q<T, DH>(P, bh, s_tok, q_reg, lane);
+    }
     TokenRegs tok;
     if (token_wave) tok = token_load<T, DH, XFORM>(P, bh, s_tok, lane);
 
@@ -1437,6 +1511,7 @@ __global__ void __launch_bounds__(NW * 64) ffa_scores_kernel(HOT_PARAMS_DECL, co
     constexpr int NCH = G::NCH;
     __shared__ float s_m[NW], s_l[NW];
     __shared__ TokenLds<T, DH> s_tok;
+    __shared__ AngleLds<T, DH, XFORM> s_ang;
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const unsigned pair = pair_of(P, blockIdx.x);
@@ -1451,9 +1526,17 @@ __global__ void __launch_bounds__(NW * 64) ffa_scores_kernel(HOT_PARAMS_DECL, co
 
     const bool token_wave = split == P.n_splits - 1 && wave == 0;
     uint4 q_reg[G::QREG];
-    // With a transform, wave 0 of every piece transforms q; the piece that holds the token also k and v.
-    const bool q_in_lds = setup_q<T, DH, XFORM>(P, bh, tlen, first, /*compute=*/wave == 0,
-                                                /*with_kv=*/token_wave, s_tok, q_reg, lane);
+    // With a transform, wave 0 of every piece publishes the angles; in the piece that holds the token it
+    // also transforms k and v.
+    bool q_in_lds = true;
+    if constexpr (XFORM) {
+        RawToken<T, DH> raw;
+        xform_begin<T, DH>(raw, P, bh, tlen, first, /*needs_q=*/true, /*publisher=*/wave == 0, /*with_kv=*/token_wave, s_ang,
+                           lane);
+        xform_end<T, DH>(raw, P, true, wave == 0, token_wave, s_tok, s_ang, lane);
+    } else {
+        q_in_lds = setup_q<T, DH>(P, bh, s_tok, q_reg, lane);
+    }
     TokenRegs tok;
     if (token_wave) tok = token_load<T, DH, XFORM>(P, bh, s_tok, lane);
 
