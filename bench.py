@@ -115,6 +115,7 @@ class Workload:
         self.ws = torch.zeros(nbytes, dtype=torch.uint8, device=dev)
         self.ws_bytes = nbytes
         self._plans = {}
+        self.transform = None     # a capi.TokenTransform: the step then goes through ffa_attention_ex
         torch.cuda.synchronize()
 
     @staticmethod
@@ -150,6 +151,16 @@ class Workload:
         """One step through the C ABI (no allocation, no sync)."""
         t = self.t_of(i)
         r, l = i % self.ring, i % self.layers
+        if self.transform is not None:
+            rc = self.lib.ffa_attention_ex(
+                self.precision, self.B, self.H, self.Dh, self.Lmax, self.scale, t,
+                self.q[r].data_ptr(), self.k[r].data_ptr(), self.v[r].data_ptr(),
+                self.kc[l].data_ptr(), self.vc[l].data_ptr(), self.out[r].data_ptr(), None, 0.0,
+                C.byref(self.plan_for(t)), 1, C.byref(self.transform), None, self.ws.data_ptr(), self.ws_bytes,
+                stream_ptr)
+            if rc != 0:
+                raise RuntimeError(f"ffa_attention_ex failed: {self.capi.status_string(rc)}")
+            return
         rc = self.fn_attn(
             self.B, self.H, self.Dh, self.Lmax, self.scale, t,
             self.q[r].data_ptr(), self.k[r].data_ptr(), self.v[r].data_ptr(),
@@ -644,13 +655,31 @@ def run_hf_end_to_end(family="opt", B=None, prompt=None, new_tokens=128):
                         f"{new_tokens} {how} tokens; per-token time excludes the prompt pass", **res}
 
 
-def measure_row(name, use_default=False, steps=32, eager=True):
+def measure_row(name, use_default=False, steps=32, eager=True, rotary_dim=0):
     """One short row of the headline measurement for another workload: `steps` launches that
     sample its whole decode, repeated to a region of at least MIN_REGION_MS; graph replay
-    (median of 5) and, beside it, the eager C-ABI leg."""
+    (median of 5) and, beside it, the eager C-ABI leg.  With `rotary_dim` the step carries the
+    rotary embedding of the new token (ffa_attention_ex); the plain step is timed beside it, the
+    two alternating, and the row reports both."""
     import torch
     wl = Workload(name, use_default=use_default, steps=steps)
     n = launches_for(wl, steps, 16)
+    if rotary_dim:
+        from fastforwardattention_amd import capi
+        tt, both = capi.TokenTransform(None, None, None, rotary_dim, 0.0), {False: [], True: []}
+        for _ in range(3):
+            for on in (False, True):
+                wl.transform = tt if on else None
+                both[on].append(median(run_graph(wl, n, replays=3)) * 1e3 / n)
+        plain_us, us = median(both[False]), median(both[True])
+        mb = wl.mean_bytes()
+        row = {"workload": name, "token_transform": f"rotary embedding over {rotary_dim} of {wl.Dh} dims", "B": wl.B,
+               "H": wl.H, "Dh": wl.Dh, "dtype": wl.dtype, "t_range": list(wl.t_range()), "timed_launches": n,
+               "us_per_step": round(us, 2), "plain_us_per_step": round(plain_us, 2),
+               "transform_costs_us": round(us - plain_us, 2), "GBps": round(mb / us / 1e3, 1)}
+        del wl
+        torch.cuda.empty_cache()
+        return row
     us = median(run_graph(wl, n)) * 1e3 / n
     mb = wl.mean_bytes()
     row = {"workload": name, "use_default_kernel_launch": use_default, "B": wl.B, "H": wl.H, "Dh": wl.Dh,
@@ -677,6 +706,14 @@ SUITE_ROWS = [  # (workload, also with the default launch)
 ]
 
 
+TRANSFORM_ROWS = [("gptj_b8", 64), ("opt1.3b_b10", 32), ("opt1.3b_b1", 32), ("long_b1_4k", 32)]  # workload, rotary dims
+
+
+def run_transform_rows():
+    """The step with the new token's rotary embedding inside the launch, beside the plain step."""
+    return [measure_row(name, rotary_dim=rd) for name, rd in TRANSFORM_ROWS]
+
+
 def run_suite_rows(full=False):
     """The other BASELINE configurations, same method as the headline line, short rows."""
     rows = []
@@ -684,6 +721,7 @@ def run_suite_rows(full=False):
         rows.append(measure_row(name))
         if with_default:
             rows.append(measure_row(name, use_default=True, eager=False))
+    rows.extend(run_transform_rows())
     sweep = run_pruned_sweep(16, "library")
     rows.append(sweep)
     rows.append(run_pruned_sweep(1, "library"))
@@ -1032,6 +1070,8 @@ def main():
     ap.add_argument("--sweep-out", default=None, help="where --sweep-plans writes the table")
     ap.add_argument("--init-cache", action="store_true", help="only the cache-construction kernel at the BASELINE shapes")
     ap.add_argument("--pruned-sweep", action="store_true", help="only the pruned sweep (BASELINE configs[4])")
+    ap.add_argument("--transform-rows", action="store_true",
+                    help="only the rows that time the step with a rotary embedding against the plain step")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="run a plain 128 MiB copy kernel 40 times (reference for rocprofv3 --pmc FETCH_SIZE / "
                          "WRITE_SIZE scaling) and exit")
@@ -1063,6 +1103,10 @@ def main():
         return
     if args.pruned_sweep:
         run_pruned_sweeps()
+        return
+    if args.transform_rows:
+        for row in run_transform_rows():
+            print(json.dumps(row), flush=True)
         return
     if args.init_cache:
         print(json.dumps(run_init_cache_bench()))

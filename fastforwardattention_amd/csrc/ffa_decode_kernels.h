@@ -244,7 +244,7 @@ __device__ __forceinline__ void token_load_rest(RawToken<T, DH>& r, const Decode
     // Every load below is issued whatever is present (an absent operand reads q once more and
     // the value is never looked at): with a fixed number of loads in flight each wait is for the
     // operand it names, not for the last load issued.
-    const int h = bh % P.H;
+    const int h = (P.q_bias || P.k_bias || P.v_bias) ? bh % P.H : 0;  // a division: not in front of the angles for nothing
     const void* qb = P.q_bias ? P.q_bias : P.q;
     const void* kb = P.k_bias ? P.k_bias : P.q;
     const void* vb = P.v_bias ? P.v_bias : P.q;

@@ -217,8 +217,9 @@ int ffa_attention_diag(int precision, int batch_size, int head_num, int head_dim
  *              real tokens before the new one: t, or seq_lengths[b] with right padding, or
  *              t - seq_lengths[b] with left padding (the reference rotates by t alone and so
  *              supports no padded batch, attention.cu:879).  The transformed k and v are what
- *              the caches receive.  It runs as one small kernel ahead of the decode kernel on
- *              the same stream; its output lives in the workspace.
+ *              the caches receive.  It runs inside the decode launch (no kernel of its own,
+ *              no workspace): one wave per workgroup computes the angles, every wave rotates
+ *              its own copy of q, the wave that appends the token also k and v.
  *   beams      NULL = none.  Otherwise beam-search cache indirection (attention.cu:779-793,
  *              :1003, :1024-1033, :1143, :1195-1202; the reference's host code passes nullptr
  *              and beam_width 1, attention.cu:1477-1479): sample b is beam b % beam_width of
