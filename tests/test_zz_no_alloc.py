@@ -121,3 +121,45 @@ def test_static_scratch_in_a_captured_graph():
         call(None)                       # eager work between the replays
         torch.cuda.synchronize()
         assert torch.equal(out, eager)
+
+
+def _ex_pair(prec, B, H, Dh, t, bw, seed):
+    """One step with a rotary embedding, a q and k bias and a random beam table: through the static
+    scratch and through ffa_attention_ex with a workspace.  Bit-equal outputs and caches."""
+    print("static scratch with transform and beams", dict(prec=prec, B=B, H=H, Dh=Dh, t=t, bw=bw), flush=True)
+    rng, K, V = rand_inputs(seed, B, H, t, Dh, prec, kv_scale=0.5)
+    q, k, v = rand_token(rng, B, H, Dh, prec)
+    sess = CApiSession(K, V, t + 2)
+    dev, tdt = "cuda:0", sess.k_cache.dtype
+    qd, kd, vd = (torch.from_numpy(np.ascontiguousarray(x)).to(dev) for x in (q, k, v))
+    bias = [torch.from_numpy((0.25 * rng.standard_normal((H, Dh))).astype(np.float32)).to(dev).to(tdt) for _ in range(2)]
+    tt = capi.TokenTransform(bias[0].data_ptr(), bias[1].data_ptr(), None, Dh // 2, 0.0)
+    table = torch.from_numpy(rng.integers(0, bw, size=(B, t + 2)).astype(np.int32)).to(dev)
+    bi = capi.BeamIndirection(table.data_ptr(), bw)
+    kc0, vc0 = sess.k_cache.clone(), sess.v_cache.clone()
+    got = []
+    for static in (True, False):
+        sess.k_cache.copy_(kc0)
+        sess.v_cache.copy_(vc0)
+        out = torch.full((B, H, Dh), float("nan"), dtype=tdt, device=dev)
+        head = (sess.precision, B, H, Dh, sess.Lmax, 0.125, t, ptr(qd), ptr(kd), ptr(vd), ptr(sess.k_cache),
+                ptr(sess.v_cache), ptr(out), None, 0.0, None, 1, C.byref(tt), C.byref(bi))
+        if static:
+            rc = sess.lib.ffa_attention_static_scratch(*head, None)
+        else:
+            rc = sess.lib.ffa_attention_ex(*head, ptr(sess.ws), sess.ws.numel(), None)
+        assert rc == capi.FFA_OK, capi.STATUS_NAMES.get(rc, rc)
+        torch.cuda.synchronize()
+        got.append((out.cpu().numpy(), sess.k_cache.cpu().numpy(), sess.v_cache.cpu().numpy()))
+    assert np.isfinite(got[0][0].astype(np.float32)).all()
+    for a, b in zip(*got):
+        np.testing.assert_array_equal(a.view(np.uint8), b.view(np.uint8))
+    # the transform did happen: the appended key differs from the raw k
+    assert not np.array_equal(got[0][1], kc0.cpu().numpy())
+
+
+@pytest.mark.parametrize("prec", [16, 32])
+def test_static_scratch_takes_transform_and_beams(prec):
+    """Two calls in a row on the GPU's one scratch array, the second on a smaller problem."""
+    _ex_pair(prec, 4, 16, 64, 1500, 2, 11)     # split pairs: partials and counters in the scratch
+    _ex_pair(prec, 2, 4, 128, 300, 2, 12)
