@@ -1302,9 +1302,15 @@ __global__ void __launch_bounds__(NW * 64) ffa_decode_wg_kernel(HOT_PARAMS_DECL,
     __shared__ float s_red[NW];
     __shared__ unsigned s_cnt[NW];
     __shared__ TokenLds<T, DH> s_tok;
-    __shared__ AngleLds<T, DH, XFORM> s_ang;
-    __shared__ float s_qw[NW][2 * kWave];
-    __shared__ int s_qr[NW][2 * kWave];
+    // The angles of the token transform are read before the first score is written, the survivor
+    // queues are filled after the barriers that follow the last score: one piece of LDS serves
+    // both (the dynamic part may take all but 20 KiB of the CU's LDS).
+    constexpr size_t kQueueBytes = sizeof(float) * NW * 2 * kWave;
+    constexpr size_t kAngleBytes = sizeof(AngleLds<T, DH, XFORM>);
+    __shared__ __align__(16) unsigned char s_shared[2 * kQueueBytes > kAngleBytes ? 2 * kQueueBytes : kAngleBytes];
+    AngleLds<T, DH, XFORM>& s_ang = *reinterpret_cast<AngleLds<T, DH, XFORM>*>(s_shared);
+    float(*s_qw)[2 * kWave] = reinterpret_cast<float(*)[2 * kWave]>(s_shared);
+    int(*s_qr)[2 * kWave] = reinterpret_cast<int(*)[2 * kWave]>(s_shared + kQueueBytes);
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int bh = blockIdx.x;

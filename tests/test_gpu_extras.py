@@ -253,6 +253,17 @@ def test_rotary_and_bias(elem, Dh, rd, padding):
 
 
 @pytest.mark.parametrize("elem", ["f16", "f32"])
+def test_transform_in_the_one_workgroup_kernel_at_its_lds_ceiling(elem):
+    """35839 keys through a 16-wave one-workgroup plan: 140 KiB of dynamic LDS for the scores beside
+    the kernel's static LDS, in which the angles of the transform share their place with the
+    survivor queues.  Widest head, so that the static part is at its largest."""
+    L, Dh = 35839, 256
+    plan = capi.make_plan(capi.FFA_LAUNCH_WORKGROUP, 16, 1, L // 64 + 1)
+    _say("transform at the lds ceiling", elem)
+    _check_transform(elem, 1, 2, Dh, L, 64, True, "none", 77, plan=plan)
+
+
+@pytest.mark.parametrize("elem", ["f16", "f32"])
 def test_bias_only_is_exact_and_every_plan_takes_the_transform(elem):
     B, H, Dh, L = 2, 3, 64, 333
     prec = 16 if elem == "f16" else 32
