@@ -117,8 +117,11 @@ static const GridRow* nearest_grid_row(int precision, int bh, int Dh, int t, int
     double best_d = 1e30;
     for (const GridRow* r = kPlanGrid; r->precision != 0; ++r) {
         if (r->precision != precision || r->head_dim != Dh || r->pruned != pruned) continue;
+        // Within a factor of sqrt(2) both ways, in integers (no integer ratio equals sqrt(2)): the
+        // logarithms are taken for the handful of rows that pass, not for the whole class.
+        const auto within = [](long long a, long long b) { return a >= b ? a * a <= 2 * b * b : b * b <= 2 * a * a; };
+        if (!within(bh, r->pairs) || !within((long long)t + 1, (long long)r->t + 1)) continue;
         const double dp = fabs(log2((double)bh / r->pairs)), dt = fabs(log2((t + 1.0) / (r->t + 1.0)));
-        if (dp > 0.5 || dt > 0.5) continue;
         if (dp + dt < best_d) {
             best_d = dp + dt;
             best = r;
