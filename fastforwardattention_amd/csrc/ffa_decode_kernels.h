@@ -469,11 +469,19 @@ __device__ __forceinline__ float token_score(const TokenRegs& r, int lane) {
 }
 // Append k, v at slot tlen of the pair's own caches (attention.cu:901-914, :1246).
 template <typename T, int DH>
-__device__ __forceinline__ void token_store(const TokenRegs& r, char* kc_bh, char* vc_bh, int tlen, int Lmax, int lane) {
+__device__ __forceinline__ void token_store(const TokenRegs& r, char* kc_bh, char* vc_bh, int tlen, int Lmax, int lane,
+                                            bool through = false) {
     constexpr int NCH = Geo<T, DH>::NCH;
     if (lane < NCH) {
-        st16(kc_bh + ((size_t)lane * Lmax + tlen) * 16, r.k);
-        st16(vc_bh + ((size_t)tlen * NCH + lane) * 16, r.v);
+        char* kp = kc_bh + ((size_t)lane * Lmax + tlen) * 16;
+        char* vp = vc_bh + ((size_t)tlen * NCH + lane) * 16;
+        if (through) {
+            st16_through(kp, r.k);
+            st16_through(vp, r.v);
+        } else {
+            st16(kp, r.k);
+            st16(vp, r.v);
+        }
     }
 }
 
@@ -823,7 +831,8 @@ __device__ __forceinline__ void finish_piece(const DecodeParams& P, int bh, int 
             }
             Mg = Mb;
         }
-        store_out(out, d, Lg > 0.f ? o / Lg : 0.f);
+        if (P.store_through) store_out_through(out, d, Lg > 0.f ? o / Lg : 0.f);
+        else store_out(out, d, Lg > 0.f ? o / Lg : 0.f);
     }
     // Ready for the next launch on this stream (kernel boundaries order this store).
     if (lane == 0) __hip_atomic_store(&P.ws_cnt[(size_t)bh * kCounterStride], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -1035,7 +1044,7 @@ ffa_decode_split_kernel(HOT_PARAMS_DECL, const DecodeParams P_rest) {
     }  // tile waves
 
     finish_piece<T, DH, NW + 1>(P, bh, split, n_splits, acc, m_run, l_run, s_merge);
-    if (has_token) token_store<T, DH>(tok, kc_bh, vc_bh, tlen, P.Lmax, lane);
+    if (has_token) token_store<T, DH>(tok, kc_bh, vc_bh, tlen, P.Lmax, lane, P.store_through != 0);
 }
 
 // ---------------------------------------------------------------------------------------
@@ -1197,7 +1206,7 @@ ffa_decode_split_tpk_kernel(HOT_PARAMS_DECL, const DecodeParams P_rest) {
     }
     }  // tile waves
     finish_piece<T, DH, NW + 1>(P, bh, split, n_splits, acc, m_run, l_run, s_merge);
-    if (has_token) token_store<T, DH>(tok, kc_bh, vc_bh, tlen, P.Lmax, lane);
+    if (has_token) token_store<T, DH>(tok, kc_bh, vc_bh, tlen, P.Lmax, lane, P.store_through != 0);
 }
 
 // ---------------------------------------------------------------------------------------

@@ -85,6 +85,14 @@ __device__ __forceinline__ uint4 ld16(const void* p) {
 __device__ __forceinline__ void st16(void* p, const uint4& v) {
     *reinterpret_cast<uint4*>(p) = v;
 }
+// The same store written through to memory (`sc0 sc1`): nothing of it stays dirty in the L2.  In a
+// launch that consists of split pairs only -- few workgroups, a kernel that ends on a chain of
+// small stores -- this shortens the end of the kernel (B = 1 and 2 at 1000 keys: -0.1 us per
+// launch); with whole pairs in the launch it costs more than it saves (320 pairs: +0.25 us).
+__device__ __forceinline__ void st16_through(void* p, const uint4& v) {
+    u32x4_t w = {v.x, v.y, v.z, v.w};
+    asm volatile("global_store_dwordx4 %0, %1, off sc0 sc1" ::"v"(p), "v"(w) : "memory");
+}
 // Streaming store for cache construction (with ld16 on the read side: 8-10 % over plain
 // accesses; for the single appended row of a decode step the hint makes no difference).
 __device__ __forceinline__ void st16_stream(void* p, const uint4& v) {
@@ -144,6 +152,18 @@ __device__ __forceinline__ void store_out(uint16_t* out, int idx, float v) {
 }
 __device__ __forceinline__ void store_out(float* out, int idx, float v) { out[idx] = v; }
 __device__ __forceinline__ void store_out(bf16_t* out, int idx, float v) { out[idx].bits = float_to_bf16(v); }
+// Written through (see st16_through).
+__device__ __forceinline__ void store_out_through(uint16_t* out, int idx, float v) {
+    const unsigned bits = __builtin_bit_cast(uint16_t, (_Float16)v);
+    asm volatile("global_store_short %0, %1, off sc0 sc1" ::"v"(out + idx), "v"(bits) : "memory");
+}
+__device__ __forceinline__ void store_out_through(float* out, int idx, float v) {
+    asm volatile("global_store_dword %0, %1, off sc0 sc1" ::"v"(out + idx), "v"(v) : "memory");
+}
+__device__ __forceinline__ void store_out_through(bf16_t* out, int idx, float v) {
+    const unsigned bits = float_to_bf16(v);
+    asm volatile("global_store_short %0, %1, off sc0 sc1" ::"v"(out + idx), "v"(bits) : "memory");
+}
 
 // ---------------------------------------------------------------------------------------
 // The reference's pruning predicate.

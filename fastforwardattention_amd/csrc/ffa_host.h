@@ -82,6 +82,7 @@ struct DecodeParams {
     int xform;               // any bias or a rotary embedding present
     double rotary_coef;      // -2 log2(base) / rotary_dim: angle of pair z = pos * 2^(z * coef)
     int floor_probe;         // launch ffa_load_floor_kernel instead of the decode kernel
+    int store_through;       // split launch without whole pairs: outputs and appended rows are written through
 };
 
 // Carved-up workspace for a given plan.

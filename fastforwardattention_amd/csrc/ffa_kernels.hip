@@ -132,6 +132,7 @@ int launch_decode(const DecodeArgs& a, const ffa_launch_plan& plan, const Worksp
     P.rotary_dim = a.rotary_dim;
     P.xform = a.transforms_token() ? 1 : 0;
     P.floor_probe = a.floor_probe ? 1 : 0;
+    P.store_through = (plan.kind == FFA_LAUNCH_SPLIT && plan.n_splits > 1 && plan.whole_heads == 0) ? 1 : 0;
     P.rotary_coef = a.rotary_dim > 0 ? -2.0 * log2((double)a.rotary_base) / (double)a.rotary_dim : 0.0;
     // The transform is a compile-time switch of the kernels: the plain step carries none of its code.
     if (P.xform) {
