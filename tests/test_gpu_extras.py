@@ -471,12 +471,12 @@ def _check_caches_after_transforms(sess, kc, vc, n, elem):
 
 
 def test_rotary_decode_on_one_workspace_across_plan_changes():
-    """GPT-J-shaped iterative decode at B = 1 (16 heads x 256, rotary_dim 64, fp16), t = 250 -> 450,
+    """GPT-J-shaped iterative decode at B = 1 (16 heads x 256, rotary_dim 64, fp16), t = 100 -> 300,
     ONE session and ONE workspace, the library's own plan at every step.  The planner moves between
     launches that use no workspace and sequence-split launches on the way (the test asserts that
     it does), so whatever a step leaves in the workspace meets the arrival counters of a later
     step.  Reference: the token transform of attention.cu:856-882 keeps no state between calls."""
-    B, H, Dh, L, rd, elem, end = 1, 16, 256, 250, 64, "f16", 450
+    B, H, Dh, L, rd, elem, end = 1, 16, 256, 100, 64, "f16", 300
     rng, K, V, *_ = _inputs(4100, B, H, L, Dh, elem)
     sess = ExSession(K, V, end + 1, elem)
     kc, vc = _pack(K, V, end + 1, elem)
