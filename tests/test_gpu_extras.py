@@ -252,6 +252,16 @@ def test_rotary_and_bias(elem, Dh, rd, padding):
     _check_transform(elem, 2, 2, Dh, 130, rd, False, padding, 901 + Dh + rd)
 
 
+@pytest.mark.parametrize("padding", ["none", "left"])
+def test_rotary_at_the_gptj_baseline_shape(padding):
+    """BASELINE configs[3] (B = 8, 16 heads x 256, fp16) at 2000 cached keys with GPT-J's rotary
+    embedding over 64 dims, the library's own plan (four lanes per key, every pair cut in two)."""
+    _say("rotary at the gpt-j shape", padding)
+    plan = capi.plan_launch(16, 8, 16, 256, 2000)
+    assert plan.kind == capi.FFA_LAUNCH_SPLIT and plan.threads_per_key == 4 and plan.n_splits > 1
+    _check_transform("f16", 8, 16, 256, 2000, 64, False, padding, 2024)
+
+
 @pytest.mark.parametrize("elem", ["f16", "f32"])
 def test_transform_in_the_one_workgroup_kernel_at_its_lds_ceiling(elem):
     """35839 keys through a 16-wave one-workgroup plan: 140 KiB of dynamic LDS for the scores beside
