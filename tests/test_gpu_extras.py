@@ -262,6 +262,16 @@ def test_rotary_at_the_gptj_baseline_shape(padding):
     _check_transform("f16", 8, 16, 256, 2000, 64, False, padding, 2024)
 
 
+@pytest.mark.parametrize("elem", ["f16", "bf16", "f32"])
+def test_rotary_and_bias_at_the_headline_shape(elem):
+    """BASELINE configs[1] at B = 10 (320 pairs of 64) at 1100 cached keys: the hybrid launch, 256 whole
+    pairs and 64 split ones, every workgroup with a wave that publishes the angles."""
+    _say("rotary+bias at the headline shape", elem)
+    plan = capi.plan_launch(32 if elem == "f32" else 16, 10, 32, 64, 1100)
+    assert plan.kind == capi.FFA_LAUNCH_SPLIT and plan.whole_heads == 256 and plan.n_splits > 1
+    _check_transform(elem, 10, 32, 64, 1100, 32, True, "right", 2025)
+
+
 @pytest.mark.parametrize("elem", ["f16", "f32"])
 def test_transform_in_the_one_workgroup_kernel_at_its_lds_ceiling(elem):
     """35839 keys through a 16-wave one-workgroup plan: 140 KiB of dynamic LDS for the scores beside
