@@ -903,7 +903,7 @@ def candidate_plans(capi, prec, B, H, Dh, t, p, cus):
     return uniq
 
 
-GRID_T = (128, 256, 512, 1024, 2048, 4096, 8192, 16384)
+GRID_T = (128, 192, 256, 384, 512, 768, 1024, 1536, 2048, 3072, 4096, 6144, 8192, 12288, 16384)
 GRID_BH = ((1, 16), (1, 32), (2, 32), (4, 32), (8, 32), (10, 32), (16, 32), (32, 32))
 
 

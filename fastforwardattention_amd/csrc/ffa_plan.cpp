@@ -9,6 +9,8 @@
 #include <math.h>
 #include <stdlib.h>
 
+#include <vector>
+
 #include "ffa_host.h"
 
 namespace ffa {
@@ -112,11 +114,38 @@ static const GridRow kPlanGrid[] = {
     {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0.f, 0.f, 0.f}  // sentinel
 };
 
+// The rows of one (precision, head dimension, pruned) class, gathered once: a lookup walks its
+// own class (a tenth of the grid), not the whole table.
+struct GridClass {
+    int precision, head_dim, pruned;
+    std::vector<const GridRow*> rows;
+};
+static const std::vector<GridClass>& grid_classes() {
+    static const std::vector<GridClass> classes = [] {
+        std::vector<GridClass> out;
+        for (const GridRow* r = kPlanGrid; r->precision != 0; ++r) {
+            GridClass* c = nullptr;
+            for (GridClass& k : out)
+                if (k.precision == r->precision && k.head_dim == r->head_dim && k.pruned == r->pruned) c = &k;
+            if (c == nullptr) {
+                out.push_back(GridClass{r->precision, r->head_dim, r->pruned, {}});
+                c = &out.back();
+            }
+            c->rows.push_back(r);
+        }
+        return out;
+    }();
+    return classes;
+}
+
 static const GridRow* nearest_grid_row(int precision, int bh, int Dh, int t, int pruned) {
     const GridRow* best = nullptr;
     double best_d = 1e30;
-    for (const GridRow* r = kPlanGrid; r->precision != 0; ++r) {
-        if (r->precision != precision || r->head_dim != Dh || r->pruned != pruned) continue;
+    const GridClass* cls = nullptr;
+    for (const GridClass& k : grid_classes())
+        if (k.precision == precision && k.head_dim == Dh && k.pruned == pruned) cls = &k;
+    if (cls == nullptr) return nullptr;
+    for (const GridRow* r : cls->rows) {
         // Within a factor of sqrt(2) both ways, in integers (no integer ratio equals sqrt(2)): the
         // logarithms are taken for the handful of rows that pass, not for the whole class.
         const auto within = [](long long a, long long b) { return a >= b ? a * a <= 2 * b * b : b * b <= 2 * a * a; };
@@ -288,7 +317,11 @@ static int plan_by_rules(int precision, int B, int H, int Dh, int t, float p, in
     if (n_splits > cap) n_splits = cap;
     if (n_splits < 1) n_splits = 1;
     const int nch = Dh * (precision / 8) / 16;  // 16-byte chunks per key: a 64-key tile is nch x 2 KiB
-    if (whole == 0 && n_splits > 1 && (long long)ntiles * nch * (n_splits - 1) < 80ll * n_splits) n_splits = 1;
+    // A cut pays once it saves more than the merge costs: about ten 16 KiB tile-times where the
+    // whole pairs already keep half the CUs busy (2 or 3 pieces), about seven where they leave
+    // three quarters or more of them idle (32 pairs x 760 keys: 5.9 us whole, 4.6 us in 8 pieces).
+    const long long cut_cost = n_splits >= 4 ? 56 : 80;
+    if (whole == 0 && n_splits > 1 && (long long)ntiles * nch * (n_splits - 1) < cut_cost * n_splits) n_splits = 1;
     const int tps = ceil_div(ntiles, n_splits);
     n_splits = ceil_div(ntiles, tps);
     const int tpk = (nch >= 16 && bh < 2 * cus && tpk_supported(precision, Dh, 4)) ? 4 : 1;
