@@ -263,7 +263,12 @@ static int plan_by_rules(int precision, int B, int H, int Dh, int t, float p, in
         const int cap = max_splits_for(bh, t + 1);
         if (n_splits > cap) n_splits = cap;
         if (n_splits < 1) n_splits = 1;
-        const bool cut_pays = bh < cus && n_splits > 1 && ntiles * (n_splits - 1.7) >= 12.0 * n_splits;
+        // Wide rows are cut earlier (a tile of 32 chunks per key weighs two of 8 in this balance:
+        // 64 pairs x 768 keys of Dh 256 16-20 % ahead in 7 pieces), nothing below ten tiles.
+        const int nch = Dh * (precision / 8) / 16;
+        const double width = nch >= 32 ? 2.0 : nch >= 16 ? 1.3 : 1.0;
+        const bool cut_pays = bh < cus && n_splits > 1 && ntiles >= 10 &&
+                              ntiles * width * (n_splits - 1.7) >= 12.0 * n_splits;
         if (fits_wg && !cut_pays) {
             // Waves: one tile or two per wave up to 8 waves; 16 waves only for very long sequences
             // with a whole number of pairs per CU (512 pairs x 8192 keys); 4 waves when some CUs get
@@ -271,7 +276,12 @@ static int plan_by_rules(int precision, int B, int H, int Dh, int t, float p, in
             int want = ntiles <= 5 ? 4 : 8;
             if (bh % cus == 0 && ntiles >= 128) want = 16;
             if (bh > cus && bh % cus != 0) want = 4;
-            fill(plan, FFA_LAUNCH_WORKGROUP, wg_waves_for(ntiles, want), 1, ntiles);
+            int w = wg_waves_for(ntiles, want);
+            // Six or seven tiles take 8 waves, not 4 (one round instead of two: 10-12 % at 384
+            // keys), and 16 where the rows are widest and the pairs few (Dh 256: 12.5 vs 17.6 us).
+            if (ntiles > 5 && want >= 8 && w < 8 && bh <= 2 * cus) w = 8;
+            if (ntiles > 5 && ntiles < 10 && nch >= 32 && 4 * bh <= cus) w = 16;
+            fill(plan, FFA_LAUNCH_WORKGROUP, w, 1, ntiles);
             return FFA_OK;
         }
         const int tps = ceil_div(ntiles, n_splits);
@@ -312,19 +322,26 @@ static int plan_by_rules(int precision, int B, int H, int Dh, int t, float p, in
     } else {
         n_splits = cus / bh;
     }
-    if (n_splits > ceil_div(ntiles, waves)) n_splits = ceil_div(ntiles, waves);
+    const int nch = Dh * (precision / 8) / 16;  // 16-byte chunks per key: a 64-key tile is nch x 2 KiB
+    const int tpk = (nch >= 16 && bh < 2 * cus && tpk_supported(precision, Dh, 4)) ? 4 : 1;
+    // Never so many pieces that a wave is left without work: with four lanes per key a 64-key
+    // tile is four units of work (16 x 256 at 384 keys: 7.5 us in 7 pieces, 8.6 in 4, 9.8 whole).
+    const int most = ceil_div(ntiles * tpk, waves);
+    if (n_splits > most) n_splits = most;
     const int cap = max_splits_for(rest > 0 ? rest : bh, t + 1);
     if (n_splits > cap) n_splits = cap;
+    if (n_splits > ntiles) n_splits = ntiles;
     if (n_splits < 1) n_splits = 1;
-    const int nch = Dh * (precision / 8) / 16;  // 16-byte chunks per key: a 64-key tile is nch x 2 KiB
     // A cut pays once it saves more than the merge costs: about ten 16 KiB tile-times where the
     // whole pairs already keep half the CUs busy (2 or 3 pieces), about seven where they leave
     // three quarters or more of them idle (32 pairs x 760 keys: 5.9 us whole, 4.6 us in 8 pieces).
-    const long long cut_cost = n_splits >= 4 ? 56 : 80;
-    if (whole == 0 && n_splits > 1 && (long long)ntiles * nch * (n_splits - 1) < cut_cost * n_splits) n_splits = 1;
+    // Wide rows with four lanes per key: from five tiles on, and about a dozen tile-times.
+    const long long cut_cost = tpk > 1 ? 100 : n_splits >= 4 ? 56 : 80;
+    if (whole == 0 && n_splits > 1 &&
+        ((long long)ntiles * nch * (n_splits - 1) < cut_cost * n_splits || (tpk > 1 && ntiles < 5)))
+        n_splits = 1;
     const int tps = ceil_div(ntiles, n_splits);
     n_splits = ceil_div(ntiles, tps);
-    const int tpk = (nch >= 16 && bh < 2 * cus && tpk_supported(precision, Dh, 4)) ? 4 : 1;
     if (n_splits == 1) {
         // Nothing is cut: one workgroup per pair.  Below one pair per CU the idle CUs are made up
         // for with 8 waves per workgroup (160 pairs, 1000 keys: 9.3 vs 9.8 us).
