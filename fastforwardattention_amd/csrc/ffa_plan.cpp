@@ -250,9 +250,9 @@ static int plan_by_rules(int precision, int B, int H, int Dh, int t, float p, in
     if (p > 0.f) {
         // Pruning needs the global max and sum before it may touch V: either one workgroup per
         // (b,h) with the scores in LDS, or the two-pass pair of kernels cut along the sequence.
-        // The second launch and the merge of the pieces cost about a dozen tile-times (of any
-        // width), and a cut in two or three gains little, so cutting a pair into n pieces pays
-        // from ntiles (1 - 1.7/n) >= 12 on, and never with a pair or more per CU (grid sweep: 16
+        // The second launch and the merge of the pieces cost about a dozen tile-times of narrow
+        // rows, and a cut in two or three gains little, so cutting a pair into n pieces pays from
+        // ntiles width (1 - 1.7/n) >= 12 on, and never with a pair or more per CU (grid sweep: 16
         // and 32 pairs go two-pass from 1024 keys, 64 pairs from 2048, 128 pairs from 8192; at 256
         // pairs and more the one-workgroup kernel wins at every length).
         // Both kernels of the pair carry only half of a tile's loads each, so from 4096 keys on
